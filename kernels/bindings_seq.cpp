@@ -1,0 +1,342 @@
+// Torch bindings of the `_C_seq` extension: f32 residual-stream ops, short
+// causal convolution with per-sequence state, latent attention.
+// Built in-tree by kernels/build.py (hipcc --offload-arch=gfx950).
+
+#include <torch/extension.h>
+#include <ATen/hip/HIPContext.h>
+
+#include <hip/hip_bf16.h>
+
+template <typename T>
+void launch_gelu_tanh(T*, const T*, const T*, long, int, long, hipStream_t);
+template <typename T>
+void launch_embedding_scaled(float*, const long*, const T*, float, int, int,
+                             hipStream_t);
+template <typename T>
+void launch_rms_norm_stream(T*, const float*, const float*, float, float, int,
+                            int, hipStream_t);
+template <typename T>
+void launch_stream_add(float*, const T*, const T*, float, T*, long, hipStream_t);
+template <typename T>
+void launch_stream_add_rms_norm(float*, const T*, const float*, float, float,
+                                int, int, hipStream_t);
+template <typename T>
+void launch_softcap(float*, const T*, float, long, hipStream_t);
+template <typename T>
+void launch_rope_partial(T*, long, long, const long*, const float*, int, int,
+                         int, int, hipStream_t);
+template <typename T>
+void launch_latent_kv_write(const T*, const float*, float, const long*,
+                            const float*, int, T*, const long*, int, int, int,
+                            hipStream_t);
+template <typename T>
+void launch_causal_conv_state(T*, const T*, const float*, T*, const int*,
+                              const int*, const int*, int, int, int, int, int,
+                              hipStream_t);
+template <typename T>
+void launch_latent_attention(T*, long, long, const T*, long, long, const T*,
+                             long, long, const T*, const int*, int, const int*,
+                             const int*, int, const float*, float, int, int,
+                             int, int, int, int, hipStream_t);
+bool latent_prefill_mfma_usable(int rank, int rot, int block_size);
+void launch_latent_prefill_mfma(__hip_bfloat16*, long, long,
+                                const __hip_bfloat16*, long, long,
+                                const __hip_bfloat16*, long, long,
+                                const __hip_bfloat16*, const int*, int,
+                                const int*, const int*, int, const float*,
+                                float, int, int, int, int, int, int,
+                                hipStream_t);
+
+namespace {
+
+hipStream_t stream() { return at::hip::getCurrentHIPStream().stream(); }
+
+template <typename T>
+T* ptr(const torch::Tensor& t) {
+  return reinterpret_cast<T*>(t.data_ptr());
+}
+
+#define DISPATCH_F32_BF16(DTYPE, BODY)                                  \
+  switch (DTYPE) {                                                      \
+    case at::ScalarType::BFloat16: {                                    \
+      using scalar_t = __hip_bfloat16;                                  \
+      BODY;                                                             \
+      break;                                                            \
+    }                                                                   \
+    case at::ScalarType::Float: {                                       \
+      using scalar_t = float;                                           \
+      BODY;                                                             \
+      break;                                                            \
+    }                                                                   \
+    default:                                                            \
+      TORCH_CHECK(false, "this op takes float32 or bfloat16 tensors");  \
+  }
+
+void check_f32(const torch::Tensor& t, const char* what) {
+  TORCH_CHECK(t.is_cuda() && t.scalar_type() == at::ScalarType::Float &&
+                  t.is_contiguous(), what, " must be a contiguous f32 GPU tensor");
+}
+void check_i32(const torch::Tensor& t, const char* what) {
+  TORCH_CHECK(t.is_cuda() && t.scalar_type() == at::ScalarType::Int &&
+                  t.is_contiguous(), what, " must be a contiguous int32 GPU tensor");
+}
+void check_i64(const torch::Tensor& t, const char* what) {
+  TORCH_CHECK(t.is_cuda() && t.scalar_type() == at::ScalarType::Long &&
+                  t.is_contiguous(), what, " must be a contiguous int64 GPU tensor");
+}
+
+void gelu_tanh(torch::Tensor out, torch::Tensor x,
+               c10::optional<torch::Tensor> mul) {
+  TORCH_CHECK(x.is_cuda() && x.is_contiguous() && out.is_contiguous());
+  TORCH_CHECK(out.scalar_type() == x.scalar_type() && out.numel() == x.numel());
+  const int cols = x.size(-1);
+  long mul_stride = 0;
+  if (mul.has_value()) {
+    const auto& m = mul.value();
+    TORCH_CHECK(m.dim() == 2 && x.dim() == 2 && m.size(0) == x.size(0) &&
+                m.size(1) == cols && m.stride(1) == 1 &&
+                m.scalar_type() == x.scalar_type(), "gelu_tanh: bad mul");
+    mul_stride = m.stride(0);
+  }
+  DISPATCH_F32_BF16(x.scalar_type(), {
+    launch_gelu_tanh<scalar_t>(
+        ptr<scalar_t>(out), ptr<scalar_t>(x),
+        mul.has_value() ? ptr<scalar_t>(mul.value()) : nullptr, mul_stride,
+        cols, x.numel(), stream());
+  });
+}
+
+void embedding_scaled(torch::Tensor out, torch::Tensor ids, torch::Tensor table,
+                      double scale) {
+  check_f32(out, "out");
+  check_i64(ids, "ids");
+  TORCH_CHECK(table.is_cuda() && table.is_contiguous() && table.dim() == 2);
+  TORCH_CHECK(out.size(0) == ids.numel() && out.size(1) == table.size(1));
+  DISPATCH_F32_BF16(table.scalar_type(), {
+    launch_embedding_scaled<scalar_t>(ptr<float>(out), ptr<long>(ids),
+                                      ptr<scalar_t>(table), (float)scale,
+                                      (int)ids.numel(), (int)table.size(1),
+                                      stream());
+  });
+}
+
+void rms_norm_stream(torch::Tensor out, torch::Tensor x, torch::Tensor weight,
+                     double eps, double offset) {
+  check_f32(x, "x");
+  check_f32(weight, "weight");
+  const int width = x.size(-1);
+  TORCH_CHECK(out.is_contiguous() && out.numel() == x.numel() &&
+              weight.numel() == width);
+  const int rows = x.numel() / width;
+  DISPATCH_F32_BF16(out.scalar_type(), {
+    launch_rms_norm_stream<scalar_t>(ptr<scalar_t>(out), ptr<float>(x),
+                                     ptr<float>(weight), (float)eps,
+                                     (float)offset, rows, width, stream());
+  });
+}
+
+void stream_add(torch::Tensor x, torch::Tensor a, c10::optional<torch::Tensor> b,
+                double mult, c10::optional<torch::Tensor> cast) {
+  check_f32(x, "x");
+  TORCH_CHECK(a.is_cuda() && a.is_contiguous() && a.numel() == x.numel());
+  if (b.has_value())
+    TORCH_CHECK(b.value().is_contiguous() && b.value().numel() == x.numel() &&
+                b.value().scalar_type() == a.scalar_type());
+  if (cast.has_value())
+    TORCH_CHECK(cast.value().is_contiguous() && cast.value().numel() == x.numel() &&
+                cast.value().scalar_type() == a.scalar_type());
+  DISPATCH_F32_BF16(a.scalar_type(), {
+    launch_stream_add<scalar_t>(
+        ptr<float>(x), ptr<scalar_t>(a),
+        b.has_value() ? ptr<scalar_t>(b.value()) : nullptr, (float)mult,
+        cast.has_value() ? ptr<scalar_t>(cast.value()) : nullptr, x.numel(),
+        stream());
+  });
+}
+
+void stream_add_rms_norm(torch::Tensor x, torch::Tensor y, torch::Tensor weight,
+                         double eps, double mult) {
+  check_f32(x, "x");
+  check_f32(weight, "weight");
+  const int width = x.size(-1);
+  TORCH_CHECK(y.is_cuda() && y.is_contiguous() && y.numel() == x.numel() &&
+              weight.numel() == width);
+  const int rows = x.numel() / width;
+  DISPATCH_F32_BF16(y.scalar_type(), {
+    launch_stream_add_rms_norm<scalar_t>(ptr<float>(x), ptr<scalar_t>(y),
+                                         ptr<float>(weight), (float)eps,
+                                         (float)mult, rows, width, stream());
+  });
+}
+
+void softcap(torch::Tensor out, torch::Tensor in, double cap) {
+  check_f32(out, "out");
+  TORCH_CHECK(in.is_cuda() && in.is_contiguous() && in.numel() == out.numel());
+  DISPATCH_F32_BF16(in.scalar_type(), {
+    launch_softcap<scalar_t>(ptr<float>(out), ptr<scalar_t>(in), (float)cap,
+                             in.numel(), stream());
+  });
+}
+
+void rope_partial(torch::Tensor x, torch::Tensor positions,
+                  torch::Tensor inv_freq, int64_t offset, int64_t rot_dims) {
+  TORCH_CHECK(x.is_cuda() && x.dim() == 3 && x.stride(2) == 1);
+  check_i64(positions, "positions");
+  check_f32(inv_freq, "inv_freq");
+  const int half = rot_dims / 2;
+  TORCH_CHECK(rot_dims % 2 == 0 && inv_freq.numel() >= half &&
+              offset >= 0 && offset + rot_dims <= x.size(2) &&
+              positions.numel() == x.size(0), "rope_partial: bad shapes");
+  if (half == 0) return;
+  DISPATCH_F32_BF16(x.scalar_type(), {
+    launch_rope_partial<scalar_t>(ptr<scalar_t>(x), x.stride(0), x.stride(1),
+                                  ptr<long>(positions), ptr<float>(inv_freq),
+                                  (int)x.size(0), (int)x.size(1), (int)offset,
+                                  half, stream());
+  });
+}
+
+void latent_kv_write(torch::Tensor dkv, torch::Tensor norm_w, double eps,
+                     torch::Tensor positions, torch::Tensor inv_freq,
+                     int64_t rot_dims, torch::Tensor cache,
+                     torch::Tensor slot_mapping) {
+  TORCH_CHECK(dkv.is_cuda() && dkv.is_contiguous() && dkv.dim() == 2);
+  check_f32(norm_w, "norm_w");
+  check_f32(inv_freq, "inv_freq");
+  check_i64(positions, "positions");
+  check_i64(slot_mapping, "slot_mapping");
+  const int rank = norm_w.numel();
+  const int rot = dkv.size(1) - rank;
+  TORCH_CHECK(rot >= 0 && rot_dims % 2 == 0 && rot_dims <= rot &&
+              inv_freq.numel() >= rot_dims / 2);
+  TORCH_CHECK(cache.is_contiguous() && cache.dim() == 3 &&
+              cache.size(2) == dkv.size(1) &&
+              cache.scalar_type() == dkv.scalar_type());
+  TORCH_CHECK(positions.numel() == dkv.size(0) &&
+              slot_mapping.numel() == dkv.size(0));
+  DISPATCH_F32_BF16(dkv.scalar_type(), {
+    launch_latent_kv_write<scalar_t>(
+        ptr<scalar_t>(dkv), ptr<float>(norm_w), (float)eps, ptr<long>(positions),
+        ptr<float>(inv_freq), (int)(rot_dims / 2), ptr<scalar_t>(cache),
+        ptr<long>(slot_mapping), (int)dkv.size(0), rank, rot, stream());
+  });
+}
+
+void causal_conv_state(torch::Tensor out, torch::Tensor h, torch::Tensor weight,
+                       torch::Tensor state, torch::Tensor loc,
+                       torch::Tensor seq_lens, torch::Tensor slots,
+                       bool add_input) {
+  TORCH_CHECK(h.is_cuda() && h.is_contiguous() && h.dim() == 2 &&
+              out.is_contiguous() && out.scalar_type() == h.scalar_type());
+  check_f32(weight, "weight");
+  check_i32(loc, "seq_start_loc");
+  check_i32(seq_lens, "seq_lens");
+  check_i32(slots, "state_slots");
+  const int width = h.size(1);
+  const int taps = weight.size(1);
+  const int nseq = seq_lens.numel();
+  TORCH_CHECK(weight.size(0) == width && loc.numel() == nseq + 1 &&
+              slots.numel() == nseq && taps >= 1);
+  TORCH_CHECK(state.is_contiguous() && state.scalar_type() == h.scalar_type() &&
+              state.dim() == 3 && state.size(1) == taps - 1 &&
+              (taps == 1 || state.size(2) == width), "conv state shape");
+  DISPATCH_F32_BF16(h.scalar_type(), {
+    launch_causal_conv_state<scalar_t>(
+        ptr<scalar_t>(out), ptr<scalar_t>(h), ptr<float>(weight),
+        ptr<scalar_t>(state), ptr<int>(loc), ptr<int>(seq_lens), ptr<int>(slots),
+        (int)h.size(0), nseq, width, taps, add_input ? 1 : 0, stream());
+  });
+}
+
+void latent_attention_common(torch::Tensor& out, torch::Tensor& q_lat,
+                             torch::Tensor& q_rot, torch::Tensor& cache,
+                             torch::Tensor& block_tables, const int* qsl,
+                             torch::Tensor& seq_lens, double scale,
+                             int64_t window,
+                             c10::optional<torch::Tensor>& sinks,
+                             bool allow_mfma) {
+  TORCH_CHECK(q_lat.is_cuda() && q_lat.dim() == 3 && q_rot.dim() == 3 &&
+              out.dim() == 3);
+  TORCH_CHECK(q_lat.stride(2) == 1 && q_rot.stride(2) == 1 && out.stride(2) == 1);
+  const int rows = q_lat.size(0), heads = q_lat.size(1), rank = q_lat.size(2);
+  const int rot = q_rot.size(2);
+  TORCH_CHECK(q_rot.size(0) == rows && q_rot.size(1) == heads &&
+              out.size(0) == rows && out.size(1) == heads && out.size(2) == rank);
+  TORCH_CHECK(cache.is_contiguous() && cache.dim() == 3 &&
+              cache.size(2) == rank + rot, "latent cache row size");
+  TORCH_CHECK(cache.scalar_type() == q_lat.scalar_type() &&
+              q_rot.scalar_type() == q_lat.scalar_type() &&
+              out.scalar_type() == q_lat.scalar_type());
+  TORCH_CHECK(rank <= 1024, "latent rank above 1024 is not supported");
+  check_i32(seq_lens, "seq_lens");
+  TORCH_CHECK(block_tables.is_cuda() &&
+              block_tables.scalar_type() == at::ScalarType::Int &&
+              block_tables.dim() == 2 && block_tables.stride(1) == 1);
+  const int nseq = seq_lens.numel();
+  TORCH_CHECK(block_tables.size(0) >= nseq);
+  TORCH_CHECK(qsl != nullptr || rows == nseq);
+  const float* sk = nullptr;
+  if (sinks.has_value()) {
+    check_f32(sinks.value(), "sinks");
+    TORCH_CHECK(sinks.value().numel() == heads);
+    sk = ptr<float>(sinks.value());
+  }
+  const int block_size = cache.size(1);
+  if (allow_mfma && q_lat.scalar_type() == at::ScalarType::BFloat16 &&
+      latent_prefill_mfma_usable(rank, rot, block_size)) {
+    using bf = __hip_bfloat16;
+    launch_latent_prefill_mfma(
+        ptr<bf>(out), out.stride(0), out.stride(1), ptr<bf>(q_lat),
+        q_lat.stride(0), q_lat.stride(1), ptr<bf>(q_rot), q_rot.stride(0),
+        q_rot.stride(1), ptr<bf>(cache), ptr<int>(block_tables),
+        (int)block_tables.stride(0), qsl, ptr<int>(seq_lens), nseq, sk,
+        (float)scale, (int)window, rows, heads, rank, rot, block_size, stream());
+    return;
+  }
+  DISPATCH_F32_BF16(q_lat.scalar_type(), {
+    launch_latent_attention<scalar_t>(
+        ptr<scalar_t>(out), out.stride(0), out.stride(1), ptr<scalar_t>(q_lat),
+        q_lat.stride(0), q_lat.stride(1), ptr<scalar_t>(q_rot), q_rot.stride(0),
+        q_rot.stride(1), ptr<scalar_t>(cache), ptr<int>(block_tables),
+        (int)block_tables.stride(0), qsl, ptr<int>(seq_lens), nseq, sk,
+        (float)scale, (int)window, rows, heads, rank, rot, block_size, stream());
+  });
+}
+
+void latent_attention_prefill(torch::Tensor out, torch::Tensor q_lat,
+                              torch::Tensor q_rot, torch::Tensor cache,
+                              torch::Tensor block_tables, torch::Tensor qsl,
+                              torch::Tensor seq_lens, double scale,
+                              int64_t window, c10::optional<torch::Tensor> sinks,
+                              int64_t max_query_len, bool generic) {
+  check_i32(qsl, "query_start_loc");
+  TORCH_CHECK(qsl.numel() == seq_lens.numel() + 1);
+  (void)max_query_len;
+  latent_attention_common(out, q_lat, q_rot, cache, block_tables, ptr<int>(qsl),
+                          seq_lens, scale, window, sinks, !generic);
+}
+
+void latent_attention_decode(torch::Tensor out, torch::Tensor q_lat,
+                             torch::Tensor q_rot, torch::Tensor cache,
+                             torch::Tensor block_tables, torch::Tensor seq_lens,
+                             double scale, int64_t window,
+                             c10::optional<torch::Tensor> sinks) {
+  latent_attention_common(out, q_lat, q_rot, cache, block_tables, nullptr,
+                          seq_lens, scale, window, sinks, false);
+}
+
+}  // namespace
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+  m.def("gelu_tanh", &gelu_tanh);
+  m.def("embedding_scaled", &embedding_scaled);
+  m.def("rms_norm_stream", &rms_norm_stream);
+  m.def("stream_add", &stream_add);
+  m.def("stream_add_rms_norm", &stream_add_rms_norm);
+  m.def("softcap", &softcap);
+  m.def("rope_partial", &rope_partial);
+  m.def("latent_kv_write", &latent_kv_write);
+  m.def("causal_conv_state", &causal_conv_state);
+  m.def("latent_attention_prefill", &latent_attention_prefill);
+  m.def("latent_attention_decode", &latent_attention_decode);
+}

@@ -1,9 +1,16 @@
-"""In-tree build of the CDNA4 HIP extension.
+"""In-tree build of the CDNA4 HIP extensions.
 
-Direct hipcc invocation (no hipify, no CUDA-compat layer): compiles every
-kernels/*.hip plus the torch bindings for gfx950 and links
-vllm_tgis_adapter_amd/_C.so.  The built .so travels with the repo snapshot to
-GPU boxes (a JIT cache would not).
+Direct hipcc invocation (no hipify, no CUDA-compat layer): compiles the
+kernel sources plus their torch bindings for gfx950 and links the shared
+objects under vllm_tgis_adapter_amd/.  The built .so files travel with the
+repo snapshot to GPU boxes (a JIT cache would not).
+
+Two extensions, so that a model only needs the one it uses:
+
+``_C``    the llama/mixtral/opt kernel set (every kernels/*.hip that is not
+          listed for another extension) + bindings.cpp
+``_C_seq`` f32-residual-stream ops, short causal convolution with per-sequence
+          state, windowed latent attention with sinks + bindings_seq.cpp
 """
 
 from __future__ import annotations
@@ -12,25 +19,47 @@ import os
 import subprocess
 import sys
 import sysconfig
+from concurrent.futures import ThreadPoolExecutor
 from pathlib import Path
 
 REPO = Path(__file__).resolve().parent.parent
 KERNELS = REPO / "kernels"
-OUT = REPO / "vllm_tgis_adapter_amd" / "_C.so"
+PKG = REPO / "vllm_tgis_adapter_amd"
 ARCH = os.environ.get("PYTORCH_ROCM_ARCH", "gfx950")
 
+_SEQ_SOURCES = ["stream_ops.hip", "canon_conv.hip", "latent_attention.hip",
+                "latent_attention_mfma.hip"]
 
-def build(verbose: bool = True, force: bool = False) -> Path:
+EXTENSIONS = {
+    "_C": dict(
+        sources=lambda: [p for p in sorted(KERNELS.glob("*.hip"))
+                         if p.name not in _SEQ_SOURCES] + [KERNELS / "bindings.cpp"],
+    ),
+    "_C_seq": dict(
+        sources=lambda: [KERNELS / n for n in _SEQ_SOURCES
+                         if (KERNELS / n).exists()] + [KERNELS / "bindings_seq.cpp"],
+    ),
+}
+OUT = PKG / "_C.so"
+
+
+def ext_path(name: str) -> Path:
+    return PKG / f"{name}.so"
+
+
+def build_ext(name: str, verbose: bool = True, force: bool = False) -> Path:
     import torch
     import torch.utils.cpp_extension as ce
 
-    sources = sorted(KERNELS.glob("*.hip")) + [KERNELS / "bindings.cpp"]
-    if OUT.exists() and not force:
-        newest_src = max(p.stat().st_mtime for p in sources + [KERNELS / "common.h"])
-        if OUT.stat().st_mtime > newest_src:
+    sources = EXTENSIONS[name]["sources"]()
+    out = ext_path(name)
+    common_h = KERNELS / "common.h"
+    if out.exists() and not force:
+        newest_src = max(p.stat().st_mtime for p in sources + [common_h])
+        if out.stat().st_mtime > newest_src:
             if verbose:
-                print(f"[kernels/build] {OUT} up to date")
-            return OUT
+                print(f"[kernels/build] {out} up to date")
+            return out
 
     include_dirs = ce.include_paths() + [sysconfig.get_path("include")]
     torch_lib = Path(torch.__file__).parent / "lib"
@@ -44,8 +73,10 @@ def build(verbose: bool = True, force: bool = False) -> Path:
         "-O3",
         "-std=c++17",
         "-fPIC",
+        # packed-f32 VALU forms are kept out of the generated code
+        "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
         f"-D_GLIBCXX_USE_CXX11_ABI={abi}",
-        "-DTORCH_EXTENSION_NAME=_C",
+        f"-DTORCH_EXTENSION_NAME={name}",
         "-DTORCH_API_INCLUDE_EXTENSION_H",
         "-D__HIP_PLATFORM_AMD__=1",
         "-DUSE_ROCM=1",
@@ -53,34 +84,60 @@ def build(verbose: bool = True, force: bool = False) -> Path:
         "-fno-gpu-rdc",
         "-Wno-unused-result",
         "-Wno-switch-bool",
+        "-Wno-unknown-warning-option",
     ] + [f"-I{d}" for d in include_dirs]
 
     objects = []
+    jobs = []
     for src in sources:
         obj = build_dir / (src.stem + ".o")
         objects.append(obj)
         if obj.exists() and not force and obj.stat().st_mtime > max(
-            src.stat().st_mtime, (KERNELS / "common.h").stat().st_mtime
+            src.stat().st_mtime, common_h.stat().st_mtime
         ):
             continue
-        cmd = ["hipcc", "-c", str(src), "-o", str(obj)] + common_flags
+        jobs.append(["hipcc", "-c", str(src), "-o", str(obj)] + common_flags)
+
+    def _run(cmd):
         if verbose:
-            print("[kernels/build]", " ".join(cmd[:4]), "...")
+            print("[kernels/build]", " ".join(cmd[:4]), "...", flush=True)
         subprocess.run(cmd, check=True)
 
+    workers = max(1, min(len(jobs), int(os.environ.get("MAX_JOBS", "0"))
+                         or min(8, os.cpu_count() or 1)))
+    if jobs:
+        with ThreadPoolExecutor(max_workers=workers) as pool:
+            list(pool.map(_run, jobs))
+
+    tmp = out.with_suffix(f".so.tmp{os.getpid()}")
     link_cmd = (
         ["hipcc", "-shared", "-fPIC"]
         + [str(o) for o in objects]
         + [f"-L{torch_lib}", "-ltorch", "-ltorch_python", "-ltorch_hip",
            "-lc10", "-lc10_hip", "-lamdhip64",
            f"-Wl,-rpath,{torch_lib}"]
-        + ["-o", str(OUT)]
+        + ["-o", str(tmp)]
     )
     if verbose:
-        print("[kernels/build] linking", OUT.name)
+        print("[kernels/build] linking", out.name, flush=True)
     subprocess.run(link_cmd, check=True)
-    return OUT
+    os.replace(tmp, out)
+    return out
+
+
+def build(verbose: bool = True, force: bool = False, only: "str | None" = None) -> Path:
+    """Build every extension (or just ``only``); returns the path of _C.so
+    (or of the single requested extension)."""
+    names = [only] if only else list(EXTENSIONS)
+    last = None
+    for n in names:
+        last = build_ext(n, verbose=verbose, force=force)
+    return last if only else OUT
 
 
 if __name__ == "__main__":
-    build(force="--force" in sys.argv)
+    only = None
+    for a in sys.argv[1:]:
+        if a.startswith("--only="):
+            only = a.split("=", 1)[1]
+    build(force="--force" in sys.argv, only=only)

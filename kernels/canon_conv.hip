@@ -1,0 +1,115 @@
+// Short depthwise causal convolution over time with per-sequence state.
+//
+//   out_t = [h_t +] sum_j w[:, j] * h_(t - taps + 1 + j)
+//
+// A step brings, for each sequence, rows [loc[s], loc[s+1]) of new inputs that
+// continue the sequence at position start = seq_len - n.  Inputs older than the
+// step's rows come from state[slot] (the last taps-1 inputs, row j holding
+// position start - (taps-1) + j); positions before 0 are zero and are never
+// read from the state, so a reused slot needs no clearing.  A second kernel on
+// the same stream advances the state past the new rows: row j of the new state
+// is position end - (taps-1) + j, taken from the step's rows or, when the step
+// is shorter than taps-1, from old state row j + n — each thread walks j
+// upwards, so it reads row j + n before that row is overwritten.
+//
+// One thread per (row, channel): consecutive threads take consecutive channels,
+// every load and store is coalesced; accumulation is f32.
+
+#include "common.h"
+
+DEVINLINE int find_seq(const int* __restrict__ loc, int nseq, int row) {
+  int lo = 0, hi = nseq;  // largest s with loc[s] <= row
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (loc[mid] <= row) lo = mid; else hi = mid;
+  }
+  return lo;
+}
+
+template <typename T>
+__global__ void causal_conv_kernel(T* __restrict__ out, const T* __restrict__ h,
+                                   const float* __restrict__ w,   // [W, taps]
+                                   const T* __restrict__ state,   // [slots, taps-1, W]
+                                   const int* __restrict__ loc,
+                                   const int* __restrict__ seq_lens,
+                                   const int* __restrict__ slots, int nseq,
+                                   int width, int taps, int add_input) {
+  const int row = blockIdx.x;
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= width) return;
+  const int s = find_seq(loc, nseq, row);
+  const int slot = slots[s];
+  const long o = (long)row * width + c;
+  if (slot < 0) {  // padding row of a captured bucket
+    out[o] = ScalarOps<T>::from_f32(0.f);
+    return;
+  }
+  const int n = loc[s + 1] - loc[s];
+  const int start = seq_lens[s] - n;
+  const int p = start + (row - loc[s]);
+  const T* st = state + (long)slot * (taps - 1) * width;
+  float acc = add_input ? ScalarOps<T>::to_f32(h[o]) : 0.f;
+  for (int j = 0; j < taps; ++j) {
+    const int pj = p - (taps - 1) + j;
+    if (pj < 0) continue;
+    float v;
+    if (pj >= start)
+      v = ScalarOps<T>::to_f32(h[(long)(loc[s] + pj - start) * width + c]);
+    else
+      v = ScalarOps<T>::to_f32(st[(long)(pj - (start - (taps - 1))) * width + c]);
+    acc += w[c * taps + j] * v;
+  }
+  out[o] = ScalarOps<T>::from_f32(acc);
+}
+
+template <typename T>
+__global__ void conv_state_update_kernel(T* __restrict__ state,
+                                         const T* __restrict__ h,
+                                         const int* __restrict__ loc,
+                                         const int* __restrict__ seq_lens,
+                                         const int* __restrict__ slots,
+                                         int width, int taps) {
+  const int s = blockIdx.x;
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= width) return;
+  const int slot = slots[s];
+  if (slot < 0) return;
+  const int n = loc[s + 1] - loc[s];
+  if (n <= 0) return;
+  const int end = seq_lens[s];
+  const int start = end - n;
+  T* st = state + (long)slot * (taps - 1) * width;
+  for (int j = 0; j < taps - 1; ++j) {
+    const int pj = end - (taps - 1) + j;
+    T v = ScalarOps<T>::from_f32(0.f);
+    if (pj >= start)
+      v = h[(long)(loc[s] + pj - start) * width + c];
+    else if (pj >= 0)
+      v = st[(long)(j + n) * width + c];
+    st[(long)j * width + c] = v;
+  }
+}
+
+template <typename T>
+void launch_causal_conv_state(T* out, const T* h, const float* w, T* state,
+                              const int* loc, const int* seq_lens,
+                              const int* slots, int rows, int nseq, int width,
+                              int taps, int add_input, hipStream_t stream) {
+  const int block = 256;
+  dim3 g1(rows, (width + block - 1) / block);
+  causal_conv_kernel<T><<<g1, block, 0, stream>>>(
+      out, h, w, state, loc, seq_lens, slots, nseq, width, taps, add_input);
+  if (taps > 1) {
+    dim3 g2(nseq, (width + block - 1) / block);
+    conv_state_update_kernel<T><<<g2, block, 0, stream>>>(
+        state, h, loc, seq_lens, slots, width, taps);
+  }
+}
+
+template void launch_causal_conv_state<float>(float*, const float*, const float*,
+                                              float*, const int*, const int*,
+                                              const int*, int, int, int, int,
+                                              int, hipStream_t);
+template void launch_causal_conv_state<__hip_bfloat16>(
+    __hip_bfloat16*, const __hip_bfloat16*, const float*, __hip_bfloat16*,
+    const int*, const int*, const int*, int, int, int, int, int, hipStream_t);

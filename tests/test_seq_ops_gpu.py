@@ -1,0 +1,158 @@
+"""HIP kernels of the `_C_seq` extension against the plain PyTorch reference of
+the same op (f32 and bf16 storage; odd sizes included)."""
+
+from __future__ import annotations
+
+import pytest
+import torch
+
+from vllm_tgis_adapter_amd import ops
+from vllm_tgis_adapter_amd.ops import reference as ref
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def _tol(dtype):
+    return dict(atol=2e-5, rtol=2e-5) if dtype == torch.float32 else dict(atol=2e-2, rtol=2e-2)
+
+
+@pytest.fixture(autouse=True)
+def _need_ext():
+    assert torch.cuda.is_available()
+    assert ops.has_native_seq(), "_C_seq must be built"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_elementwise_and_norms(dtype):
+    g = torch.Generator().manual_seed(0)
+    t, w = 37, 200
+    x = torch.randn(t, w, generator=g) * 3
+    a = torch.randn(t, w, generator=g).to(dtype)
+    b = torch.randn(t, w, generator=g).to(dtype)
+    wt = torch.randn(w, generator=g) * 0.2
+    xd, ad, bd, wd = x.cuda(), a.cuda(), b.cuda(), wt.cuda()
+
+    torch.testing.assert_close(
+        ops.rms_norm_stream(xd, wd, 1e-6, 1.0, dtype).cpu().float(),
+        ref.rms_norm_stream(x, wt, 1e-6, 1.0, dtype).float(), **_tol(dtype))
+    torch.testing.assert_close(
+        ops.gelu_tanh(ad).cpu().float(), ref.gelu_tanh(a).float(), **_tol(dtype))
+    mul = torch.randn(t, 3 * w, generator=g).to(dtype)
+    torch.testing.assert_close(
+        ops.gelu_tanh(ad, mul.cuda()[:, w:2 * w]).cpu().float(),
+        ref.gelu_tanh(a, mul[:, w:2 * w]).float(), **_tol(dtype))
+
+    x1, x2 = x.clone(), xd.clone()
+    c1 = ref.stream_add(x1, a, b, 0.7, dtype)
+    c2 = ops.stream_add(x2, ad, bd, 0.7, dtype)
+    torch.testing.assert_close(x2.cpu(), x1, atol=1e-5, rtol=1e-5)
+    torch.testing.assert_close(c2.cpu().float(), c1.float(), **_tol(dtype))
+    assert ops.stream_add(x2, ad, None, 0.5) is None
+    ref.stream_add(x1, a, None, 0.5, None)
+    torch.testing.assert_close(x2.cpu(), x1, atol=1e-5, rtol=1e-5)
+
+    ref.stream_add_rms_norm(x1, a, wt, 1e-6, 0.7)
+    ops.stream_add_rms_norm(x2, ad, wd, 1e-6, 0.7)
+    torch.testing.assert_close(x2.cpu(), x1, atol=2e-5, rtol=1e-5)
+
+    torch.testing.assert_close(
+        ops.softcap(ad * 10, 15.0).cpu(), ref.softcap(a * 10, 15.0), atol=1e-5, rtol=1e-5)
+    ids = torch.randint(0, t, (50,), generator=g)
+    torch.testing.assert_close(
+        ops.embedding_scaled(ids.cuda(), ad, 3.5).cpu(), ref.embedding_scaled(ids, a, 3.5))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("taps", [1, 2, 3, 5])
+def test_causal_conv_state(dtype, taps):
+    g = torch.Generator().manual_seed(taps)
+    w = 72
+    wt = torch.randn(w, taps, generator=g) * 0.5
+    state = torch.randn(6, taps - 1, w, generator=g).to(dtype)  # stale garbage
+    # sequences: fresh start (3 rows), continuing (1 row), continuing (7 rows),
+    # a start shorter than the taps, a padding row (slot -1)
+    loc = torch.tensor([0, 3, 4, 11, 12, 13], dtype=torch.int32)
+    lens = torch.tensor([3, 9, 20, 1, 0], dtype=torch.int32)
+    slots = torch.tensor([4, 0, 2, 5, -1], dtype=torch.int32)
+    h = torch.randn(13, w, generator=g).to(dtype)
+    s1, s2 = state.clone(), state.cuda()
+    o1 = ref.causal_conv_state(h[:12], wt, s1, loc[:5], lens[:4], slots[:4], True)
+    o2 = ops.causal_conv_state(h.cuda(), wt.cuda(), s2, loc.cuda(), lens.cuda(),
+                               slots.cuda(), True)
+    torch.testing.assert_close(o2.cpu()[:12].float(), o1.float(), **_tol(dtype))
+    assert float(o2[12].abs().max()) == 0.0
+    for sl, ln in zip(slots[:4].tolist(), lens[:4].tolist()):
+        keep = min(ln, taps - 1)   # rows before the sequence's start are free
+        if keep:
+            torch.testing.assert_close(s2.cpu()[sl, taps - 1 - keep:].float(),
+                                       s1[sl, taps - 1 - keep:].float(), **_tol(dtype))
+    torch.testing.assert_close(s2.cpu()[1], state[1])   # untouched slot
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rope_and_latent_write(dtype):
+    g = torch.Generator().manual_seed(3)
+    t, nh, d, r, rank = 19, 3, 24, 16, 40
+    q = torch.randn(t, nh, d + r, generator=g).to(dtype)
+    pos = torch.randint(0, 5000, (t,), generator=g)
+    inv = torch.tensor([10000.0 ** (-2 * i / 12) for i in range(6)])
+    q1, q2 = q.clone(), q.cuda()
+    ref.rope_partial(q1, pos, inv, d, 12)
+    ops.rope_partial(q2, pos.cuda(), inv.cuda(), d, 12)
+    torch.testing.assert_close(q2.cpu().float(), q1.float(), **_tol(dtype))
+
+    dkv = torch.randn(t, rank + r, generator=g).to(dtype)
+    nw = torch.randn(rank, generator=g)
+    c1 = torch.zeros(8, 4, rank + r, dtype=dtype)
+    c2 = c1.cuda()
+    slots = torch.randperm(32, generator=g)[:t]
+    slots[5] = -1
+    ref.latent_kv_write(dkv, nw, 1e-6, pos, inv, 12, c1, slots)
+    ops.latent_kv_write(dkv.cuda(), nw.cuda(), 1e-6, pos.cuda(), inv.cuda(), 12, c2,
+                        slots.cuda())
+    torch.testing.assert_close(c2.cpu().float(), c1.float(), **_tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rank,rot,window", [(40, 16, 7), (96, 64, 24), (130, 6, 0),
+                                             (300, 20, 300)])
+def test_latent_attention(dtype, rank, rot, window):
+    g = torch.Generator().manual_seed(rank)
+    nh, bs, nb = 3, 8, 80
+    cache = torch.randn(nb, bs, rank + rot, generator=g).to(dtype)
+    # portions: (context incl. portion, portion length)
+    seqs = [(5, 5), (300, 17), (41, 2), (290, 290 if window == 0 else 9)]
+    perm = torch.randperm(nb, generator=g).tolist()
+    tables = torch.zeros(len(seqs), nb, dtype=torch.int32)
+    k = 0
+    for i, (ctx, _) in enumerate(seqs):
+        n = (ctx + bs - 1) // bs
+        tables[i, :n] = torch.tensor(perm[k:k + n] if k + n <= nb else perm[:n])
+        k = (k + n) % nb if k + n <= nb else n
+    qsl = torch.tensor([0] + list(torch.tensor([n for _, n in seqs]).cumsum(0)), dtype=torch.int32)
+    lens = torch.tensor([c for c, _ in seqs], dtype=torch.int32)
+    t = int(qsl[-1])
+    scale = 0.3 / (rank + rot) ** 0.5
+    q_lat = torch.randn(nh, t, rank, generator=g).to(dtype).transpose(0, 1)  # strided
+    q_full = torch.randn(t, nh, 8 + rot, generator=g).to(dtype)
+    q_rot = q_full[:, :, 8:]
+    sinks = torch.randn(nh, generator=g)
+    want = ref.latent_attention(q_lat, q_rot, cache, tables, qsl, lens, scale, window, sinks)
+    out = torch.empty(nh, t, rank, dtype=dtype, device="cuda").transpose(0, 1)
+    ops.latent_attention_prefill(
+        q_lat.cuda(), q_rot.cuda(), cache.cuda(), tables.cuda(), qsl.cuda(), lens.cuda(),
+        scale, window, sinks.cuda(), max(n for _, n in seqs), out=out)
+    torch.testing.assert_close(out.cpu().float(), want.float(), **_tol(dtype))
+
+    # decode: the last row of every sequence alone
+    rows = (qsl[1:] - 1).long()
+    out_d = torch.empty(len(seqs), nh, rank, dtype=dtype, device="cuda")
+    ops.latent_attention_decode(
+        q_lat[rows].cuda(), q_rot[rows].cuda(), cache.cuda(), tables.cuda(), lens.cuda(),
+        scale, window, None, out=out_d)
+    want_d = ref.latent_attention(
+        q_lat[rows], q_rot[rows], cache, tables,
+        torch.arange(len(seqs) + 1, dtype=torch.int32), lens, scale, window, None)
+    torch.testing.assert_close(out_d.cpu().float(), want_d.float(), **_tol(dtype))

@@ -155,6 +155,10 @@ class ModelConfig:
 
 
 def _from_hf_config(model: str, hf: dict) -> ModelConfig:
+    if hf.get("architecture") == "Dolodra":
+        from ..models.dolodra import model_config_from_json
+
+        return model_config_from_json(model, hf)
     arch_list = hf.get("architectures") or []
     arch = "llama"
     if any("Mixtral" in a for a in arch_list):

@@ -23,7 +23,8 @@ _BUCKETS = [1, 2, 4, 8, 16, 24, 32, 48, 64, 96, 128, 192, 256, 384, 512, 768, 10
 
 class DecodeGraphRunner:
     def __init__(self, model, kv_caches, model_config, block_size: int,
-                 max_num_seqs: int, max_model_len: int, device: str):
+                 max_num_seqs: int, max_model_len: int, device: str,
+                 with_seq_state: bool = False):
         self.model = model
         self.kv_caches = kv_caches
         self.device = device
@@ -42,6 +43,11 @@ class DecodeGraphRunner:
         self.in_block_tables = torch.zeros(
             (bmax, self.max_blocks), dtype=torch.int32, device=dev
         )
+        # per-sequence state slots (models with layer state); padding rows
+        # carry -1 and are skipped by the state kernels
+        self.with_seq_state = with_seq_state
+        self.in_state_slots = torch.full((bmax,), -1, dtype=torch.int32, device=dev)
+        self.in_seq_loc = torch.arange(bmax + 1, dtype=torch.int32, device=dev)
         self.out_logits: dict[int, torch.Tensor] = {}
         self.graphs: dict[int, torch.cuda.CUDAGraph] = {}
         self._pool = None
@@ -61,6 +67,9 @@ class DecodeGraphRunner:
             decode_seq_lens=self.in_seq_lens[:b],
             decode_block_tables=self.in_block_tables[:b],
             max_decode_seq_len=0,
+            seq_start_loc=self.in_seq_loc[:b + 1] if self.with_seq_state else None,
+            seq_lens=self.in_seq_lens[:b] if self.with_seq_state else None,
+            state_slots=self.in_state_slots[:b] if self.with_seq_state else None,
         )
 
     @torch.inference_mode()
@@ -94,7 +103,8 @@ class DecodeGraphRunner:
         return None
 
     @torch.inference_mode()
-    def run(self, ids, pos, slots, seq_lens, block_tables) -> torch.Tensor:
+    def run(self, ids, pos, slots, seq_lens, block_tables,
+            state_slots=None) -> torch.Tensor:
         """All tensors device-resident; returns logits rows [n, vocab]."""
         n = ids.shape[0]
         b = self.bucket_for(n)
@@ -105,6 +115,9 @@ class DecodeGraphRunner:
         self.in_slots[n:b].fill_(-1)
         self.in_seq_lens[:n].copy_(seq_lens)
         self.in_seq_lens[n:b].zero_()
+        if self.with_seq_state:
+            self.in_state_slots[:n].copy_(state_slots)
+            self.in_state_slots[n:b].fill_(-1)
         w = block_tables.shape[1]
         self.in_block_tables[:n, :w].copy_(block_tables)
         if w < self.max_blocks:

@@ -38,7 +38,22 @@ class LLMEngine:
             num_blocks, config.cache_config.block_size,
             enable_prefix_caching=config.cache_config.enable_prefix_caching,
         )
-        self.scheduler = Scheduler(config.scheduler_config, self.block_manager)
+        self.state_manager = None
+        if self.worker.uses_seq_state:
+            # layer state is neither shared between requests nor rolled back
+            if config.cache_config.enable_prefix_caching:
+                raise ValueError(
+                    "prefix caching is not available for models with "
+                    "per-sequence layer state")
+            if config.speculative_model:
+                raise ValueError(
+                    "speculative decoding is not available for models with "
+                    "per-sequence layer state")
+            from .state_manager import StateSlotManager
+
+            self.state_manager = StateSlotManager(self.worker.num_state_slots)
+        self.scheduler = Scheduler(config.scheduler_config, self.block_manager,
+                                   self.state_manager)
         self.detokenizer = Detokenizer(self.tokenizer)
         self.stop_checker = StopChecker(self.model_config.max_model_len)
         self.eos_token_id = self.tokenizer.eos_token_id
@@ -445,6 +460,45 @@ class LLMEngine:
             1.0 - self.block_manager.num_free_blocks / max(1, self.block_manager.num_blocks)
         )
         return outputs
+
+    # ------------------------------------------------------------------
+    # Trace replay: the caller dictates which tokens every request runs in
+    # a step and which logits it wants back; nothing is sampled.  Requests,
+    # cache blocks, state slots, the step batch and the forward are the ones
+    # generation uses.
+    def replay_step(self, entries: "list[tuple[str, list[int], list[int]]]",
+                    finished: "list[str]" = ()):
+        """entries: (request id, next tokens, places among them whose logits
+        are wanted).  Returns the wanted logits [rows, vocab] (f32, in entry
+        order) or None.  ``finished`` requests give back cache and state
+        after the step."""
+        from .scheduler import ScheduledItem  # noqa: F401
+
+        if self._deferred is not None:
+            raise RuntimeError("replay_step cannot interleave with pipelined steps")
+        plan = []
+        wants = {}
+        for rid, tokens, want in entries:
+            req = self.scheduler.get_request(rid)
+            if req is None:
+                req = self.add_request(rid, None, list(tokens),
+                                       SamplingParams(temperature=0.0, max_tokens=1))
+            else:
+                req.prompt_token_ids.extend(tokens)
+            plan.append((req, len(tokens)))
+            wants[id(req)] = list(want)
+        sched = self.scheduler.schedule_explicit(plan)
+        for it in sched.items:
+            it.samples = False
+            it.logit_offsets = wants.get(id(it.request)) or None
+        logits = self.worker.execute_replay(sched)
+        for it in sched.items:
+            it.request.num_computed_tokens += it.num_new_tokens
+        for rid in finished:
+            req = self.scheduler.get_request(rid)
+            if req is not None:
+                self.scheduler.finish_request(req)
+        return logits
 
     def shutdown(self) -> None:
         self.worker.stop_workers()

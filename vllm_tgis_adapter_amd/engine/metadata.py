@@ -9,6 +9,7 @@ decode kernel over the rest without re-gathering.
 from __future__ import annotations
 
 from dataclasses import dataclass
+from typing import Optional
 
 import torch
 
@@ -32,6 +33,14 @@ class AttnMetadata:
     decode_seq_lens: torch.Tensor      # [nd] int32 device
     decode_block_tables: torch.Tensor  # [nd, max_blocks] int32 device
     max_decode_seq_len: int
+
+    # Every sequence of the step, prefill chunks first and then the decoding
+    # ones, for layers that carry per-sequence state (None when the model has
+    # none): rows of each sequence's new tokens, its length including them,
+    # and its state slot (-1 = padding row of a captured decode bucket).
+    seq_start_loc: Optional[torch.Tensor] = None   # [ns+1] int32 device
+    seq_lens: Optional[torch.Tensor] = None        # [ns] int32 device
+    state_slots: Optional[torch.Tensor] = None     # [ns] int32 device
 
     @property
     def num_tokens(self) -> int:

@@ -69,6 +69,8 @@ class Request:
         # KV bookkeeping
         self.block_ids: list[int] = []
         self.num_computed_tokens = 0  # tokens whose KV is in cache
+        # slot of the per-sequence layer state (models that carry one)
+        self.state_slot: Optional[int] = None
         # prefix-caching state (block_manager.match_prefix/register_prefix)
         self.prefix_key = None
         self.registered_blocks = 0

@@ -34,6 +34,9 @@ class ScheduledItem:
     request: Request
     num_new_tokens: int  # tokens whose KV is computed this step
     samples: bool        # True if this step produces a sampled token
+    # places within this portion whose logits the caller wants returned
+    # (trace replay); the rows follow all others in the step's logits
+    logit_offsets: Optional[list] = None
 
 
 @dataclass
@@ -51,9 +54,12 @@ class SchedulerOutput:
 
 
 class Scheduler:
-    def __init__(self, config: SchedulerConfig, block_manager: BlockManager):
+    def __init__(self, config: SchedulerConfig, block_manager: BlockManager,
+                 state_manager=None):
         self.config = config
         self.block_manager = block_manager
+        # StateSlotManager for models with per-sequence layer state, else None
+        self.state_manager = state_manager
         self.waiting: deque[Request] = deque()
         self.running: list[Request] = []
         self._requests: dict[str, Request] = {}
@@ -75,9 +81,15 @@ class Scheduler:
                 self.waiting.remove(req)
             except ValueError:
                 pass
-        self.block_manager.free(req)
+        self._release(req)
         self._requests.pop(request_id, None)
         return req
+
+    def _release(self, req: Request) -> None:
+        """Give back the request's cache blocks and its state slot."""
+        self.block_manager.free(req)
+        if self.state_manager is not None:
+            self.state_manager.free(req)
 
     def get_request(self, request_id: str) -> Optional[Request]:
         return self._requests.get(request_id)
@@ -89,7 +101,7 @@ class Scheduler:
         """Called by the engine after stop-condition checks."""
         if req in self.running:
             self.running.remove(req)
-        self.block_manager.free(req)
+        self._release(req)
         self._requests.pop(req.request_id, None)
 
     # ------------------------------------------------------------------
@@ -162,6 +174,8 @@ class Scheduler:
             if not self.block_manager.can_grow_to(req, target_tokens):
                 # Don't preempt running work to admit new work.
                 break
+            if self.state_manager is not None and not self.state_manager.allocate(req):
+                break  # every state slot is held by a running request
             self.waiting.popleft()
             self.block_manager.grow_to(req, target_tokens)
             now = time.time()
@@ -175,6 +189,32 @@ class Scheduler:
 
         return out
 
+    def schedule_explicit(self, plan: "list[tuple[Request, int]]") -> SchedulerOutput:
+        """One step whose portions are dictated by the caller (trace replay,
+        tests): every (request, n) runs the request's next n tokens.  Cache
+        blocks and state slots come from the same managers as in schedule();
+        nothing is preempted — a plan that does not fit raises."""
+        out = SchedulerOutput()
+        for req, n in plan:
+            if n <= 0:
+                continue
+            if req.num_computed_tokens + n > req.num_tokens:
+                raise ValueError("portion runs past the request's tokens")
+            if req not in self.running:
+                try:
+                    self.waiting.remove(req)
+                except ValueError:
+                    pass
+                if self.state_manager is not None and not self.state_manager.allocate(req):
+                    raise RuntimeError("no free state slot")
+                req.status = RequestStatus.RUNNING
+                self.running.append(req)
+            target = req.num_computed_tokens + n
+            if not self.block_manager.grow_to(req, target):
+                raise RuntimeError("cache pool exhausted")
+            out.items.append(ScheduledItem(req, n, target == req.num_tokens))
+        return out
+
     # ------------------------------------------------------------------
     def _pick_victim(self, exclude: Request) -> Optional[Request]:
         for req in reversed(self.running):
@@ -184,7 +224,7 @@ class Scheduler:
 
     def _preempt(self, req: Request, out: SchedulerOutput) -> None:
         self.running.remove(req)
-        self.block_manager.free(req)
+        self._release(req)
         # Recompute-from-scratch preemption: KV is rebuilt on re-admission
         # (already-generated tokens are recomputed like prompt tokens).
         req.num_computed_tokens = 0

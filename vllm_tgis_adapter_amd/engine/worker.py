@@ -123,6 +123,7 @@ def pack_batch(batch: dict) -> tuple[np.ndarray, np.ndarray]:
         dt.reshape(-1),
         np.asarray(batch["logit_rows"], dtype=np.int64),
         np.asarray(lora, dtype=np.int64),
+        np.asarray(batch.get("state_slots") or [], dtype=np.int64),
     ]
     header = np.array(
         [batch["num_sample_rows"], len(batch["qsl"]),
@@ -144,7 +145,7 @@ def unpack_batch(header: np.ndarray, payload: np.ndarray) -> dict:
         arrs.append(payload[off:off + n])
         off += n
     (token_ids, positions, slot_mapping, qsl, pf_lens, pf_flat, dec_lens,
-     dec_flat, logit_rows, lora) = arrs
+     dec_flat, logit_rows, lora, state_slots) = arrs
     return dict(
         token_ids=token_ids,
         positions=positions,
@@ -159,6 +160,7 @@ def unpack_batch(header: np.ndarray, payload: np.ndarray) -> dict:
         logit_rows=logit_rows.tolist(),
         num_sample_rows=int(num_sample_rows),
         lora_ids=lora.tolist() if has_lora else None,
+        state_slots=state_slots.tolist() if len(state_slots) else None,
     )
 
 
@@ -187,6 +189,9 @@ class Worker:
             self._quantize_model(config.quantization)
 
         self.block_size = config.cache_config.block_size
+        # models with per-sequence layer state need a slot per request
+        self.uses_seq_state = bool(getattr(self.model, "uses_seq_state", False))
+        self.num_state_slots = 0
         self.kv_caches: list[tuple[torch.Tensor, torch.Tensor]] = []
         self.num_blocks = 0
         self.sampler = Sampler(self.device)
@@ -278,6 +283,8 @@ class Worker:
         """Allocate the paged KV cache; returns the number of blocks."""
         cfg = self.config
         mc = self.model_config
+        if hasattr(self.model, "allocate_caches"):
+            return self._init_model_caches()
         kv_heads_local = max(1, mc.num_kv_heads // self.tp)
         # fp8 KV cache: e4m3 storage (1 B/elem) — halves the decode HBM
         # stream and doubles block capacity in the 288 GB pool
@@ -328,6 +335,47 @@ class Worker:
         self._maybe_capture_graphs()
         return self.num_blocks
 
+    def _init_model_caches(self) -> int:
+        """Cache layout defined by the model (latent rows shared between
+        layers, per-sequence state slots): the model says what a block and a
+        slot cost and allocates both; block ids and slot ids still come from
+        the engine's managers."""
+        cfg = self.config
+        mc = self.model_config
+        if cfg.cache_config.kv_cache_dtype == "fp8":
+            raise ValueError("fp8 cache storage is not available for this model")
+        self.kv_dtype = mc.dtype
+        self.num_state_slots = cfg.scheduler_config.max_num_seqs
+        block_bytes = self.model.cache_bytes_per_block(self.block_size)
+        if cfg.cache_config.num_gpu_blocks is not None:
+            self.num_blocks = cfg.cache_config.num_gpu_blocks
+        elif self.device == "cuda":
+            self._profile_peak_memory()
+            free, total = torch.cuda.mem_get_info()
+            usable = (total * cfg.cache_config.gpu_memory_utilization - (total - free)
+                      - self.num_state_slots * self.model.state_bytes_per_slot())
+            # a table row per sequence is copied every step: cap the pool at
+            # what max_num_seqs full-length sequences can hold
+            per_seq = (mc.max_model_len + self.block_size - 1) // self.block_size
+            self.num_blocks = max(64, min(int(usable // block_bytes),
+                                          per_seq * self.num_state_slots + 8))
+        else:
+            per_seq = (mc.max_model_len + self.block_size - 1) // self.block_size
+            self.num_blocks = min(8192, per_seq * cfg.scheduler_config.max_num_seqs + 8)
+        if self.tp > 1:
+            import torch.distributed as dist
+
+            t = torch.tensor(
+                [self.num_blocks], dtype=torch.int64,
+                device=self.device if self.device == "cuda" else "cpu",
+            )
+            dist.all_reduce(t, op=dist.ReduceOp.MIN)
+            self.num_blocks = int(t.item())
+        self.kv_caches = self.model.allocate_caches(
+            self.num_blocks, self.block_size, self.num_state_slots, self.device)
+        self._maybe_capture_graphs()
+        return self.num_blocks
+
     def _maybe_capture_graphs(self) -> None:
         """hipGraph-capture the decode step per batch bucket (E24).
 
@@ -366,6 +414,7 @@ class Worker:
                 self.model, self.kv_caches, self.model_config, self.block_size,
                 self.config.scheduler_config.max_num_seqs,
                 self.model_config.max_model_len, self.device,
+                with_seq_state=self.uses_seq_state,
             )
             self.graph_runner.capture()
             if self.tp > 1:
@@ -430,12 +479,18 @@ class Worker:
         )
         kv_heads_local = max(1, mc.num_kv_heads // self.tp)
         nb = (t + self.block_size - 1) // self.block_size
-        shape = (nb, self.block_size, kv_heads_local, mc.head_dim)
-        tmp_cache = [
-            (torch.zeros(shape, dtype=mc.dtype, device=self.device),
-             torch.zeros(shape, dtype=mc.dtype, device=self.device))
-            for _ in range(mc.num_layers)
-        ]
+        if hasattr(self.model, "allocate_caches"):
+            tmp_cache = self.model.allocate_caches(nb, self.block_size, 1, self.device)
+            meta.seq_start_loc = meta.prefill_query_start_loc
+            meta.seq_lens = meta.prefill_seq_lens
+            meta.state_slots = torch.zeros(1, dtype=torch.int32, device=self.device)
+        else:
+            shape = (nb, self.block_size, kv_heads_local, mc.head_dim)
+            tmp_cache = [
+                (torch.zeros(shape, dtype=mc.dtype, device=self.device),
+                 torch.zeros(shape, dtype=mc.dtype, device=self.device))
+                for _ in range(mc.num_layers)
+            ]
         hidden = self.model(ids, pos, tmp_cache, meta)
         self.model.compute_logits(hidden[-1:])
         del tmp_cache, hidden
@@ -460,6 +515,7 @@ class Worker:
         decode_tables = []
         sample_rows = []   # row in batch producing the sampled logits, per sampling item
         extra_rows = []    # rows needed for prompt logprobs
+        state_slots = []   # per sequence, in batch order (models with state)
         bs = self.block_size
 
         for it in ordered:
@@ -471,6 +527,10 @@ class Worker:
             positions.extend(range(s, e))
             lid = req.lora_request.lora_int_id if req.lora_request else 0
             lora_ids.extend([lid] * (e - s))
+            if self.uses_seq_state:
+                if req.state_slot is None:
+                    raise RuntimeError("request scheduled without a state slot")
+                state_slots.append(req.state_slot)
             for pos in range(s, e):
                 b = req.block_ids[pos // bs]
                 slot_mapping.append(b * bs + pos % bs)
@@ -488,6 +548,7 @@ class Worker:
         spec_rows: list[int] = []
         # (item, rows-in-extra-space, prompt token indices, carry_out row or None)
         prompt_lp_specs = []
+        wanted_rows: list[int] = []
         for it in ordered:
             req = it.request
             nrow = row + it.num_new_tokens
@@ -499,6 +560,9 @@ class Worker:
             elif it.samples:
                 sample_rows.append(nrow - 1)
                 sampling_items.append(it)
+            if it.logit_offsets:
+                # caller-requested logits at given places of this portion
+                wanted_rows.extend(row + o for o in it.logit_offsets)
             if (
                 req.sampling_params.prompt_logprobs is not None
                 and req.num_computed_tokens < req.num_prompt_tokens
@@ -517,7 +581,9 @@ class Worker:
                 prompt_lp_specs.append((it, lp_rows, list(range(s + 1, e)), carry_out))
             row = nrow
 
-        logit_rows_all = sample_rows + spec_rows + extra_rows
+        logit_rows_all = sample_rows + spec_rows + extra_rows + wanted_rows
+        self._wanted_row_base = len(logit_rows_all) - len(wanted_rows)
+        self._ordered_items = ordered
         batch = dict(
             token_ids=token_ids,
             positions=positions,
@@ -530,6 +596,7 @@ class Worker:
             logit_rows=logit_rows_all,
             num_sample_rows=len(sample_rows),
             lora_ids=lora_ids if any(lora_ids) else None,
+            state_slots=state_slots or None,
         )
         # host-only bookkeeping (not broadcast)
         self._sampling_items = sampling_items
@@ -577,7 +644,10 @@ class Worker:
             slots = self._h2d("slots", np.asarray(batch["slot_mapping"], dtype=np.int64), torch.int64)
             seq_lens = self._h2d("dsl", np.asarray(batch["decode_seq_lens"], dtype=np.int32), torch.int32)
             bt = self._h2d("dbt", _pad_np_tables(batch["decode_tables"]), torch.int32)
-            return self.graph_runner.run(ids, pos, slots, seq_lens, bt)
+            st = None
+            if self.uses_seq_state:
+                st = self._h2d("sts", np.asarray(batch["state_slots"], dtype=np.int32), torch.int32)
+            return self.graph_runner.run(ids, pos, slots, seq_lens, bt, st)
 
         npt = batch["qsl"][-1] if np_seqs else 0
         meta = AttnMetadata(
@@ -595,6 +665,20 @@ class Worker:
             decode_block_tables=self._h2d("dbt", _pad_np_tables(batch["decode_tables"]), torch.int32),
             max_decode_seq_len=max(batch["decode_seq_lens"], default=0),
         )
+        if self.uses_seq_state:
+            nd = len(batch["decode_seq_lens"])
+            loc = np.concatenate([
+                np.asarray(batch["qsl"] if np_seqs else [0], dtype=np.int32),
+                npt + 1 + np.arange(nd, dtype=np.int32),
+            ])
+            lens = np.concatenate([
+                np.asarray(batch["prefill_seq_lens"], dtype=np.int32),
+                np.asarray(batch["decode_seq_lens"], dtype=np.int32),
+            ])
+            meta.seq_start_loc = self._h2d("ssl", loc, torch.int32)
+            meta.seq_lens = self._h2d("sln", lens, torch.int32)
+            meta.state_slots = self._h2d(
+                "sts", np.asarray(batch["state_slots"], dtype=np.int32), torch.int32)
         from . import lora as lora_rt
 
         if batch.get("lora_ids"):
@@ -671,6 +755,40 @@ class Worker:
                         self._lt = [0.0, 0.0, 0.0, 0]
                 return _PendingStep(fused, self.sampler)
         return _DoneStep(self._execute_finish(batch, logits))
+
+    @torch.inference_mode()
+    def execute_replay(self, sched: SchedulerOutput):
+        """Run one step and return only the caller-requested logits rows, in
+        the order of sched.items (not the batch order) — f32 [rows, vocab]."""
+        batch = self.build_batch(sched)
+        if self.tp > 1:
+            import torch.distributed as dist
+
+            header, payload = pack_batch(batch)
+            tp_broadcast_object(("execute_packed", header.tolist()))
+            t = torch.from_numpy(payload).to(
+                self.device if self.device == "cuda" else "cpu")
+            dist.broadcast(t, src=0)
+        logits = self.execute_batch(batch)
+        if logits is None:
+            return None
+        wanted = logits[self._wanted_row_base:]
+        # batch order is prefill portions first, then single tokens: map the
+        # rows back to the order the caller listed its entries in
+        pos = {}
+        off = 0
+        for it in self._ordered_items:
+            n = len(it.logit_offsets or ())
+            pos[id(it)] = (off, n)
+            off += n
+        idx = []
+        for it in sched.items:
+            o, n = pos[id(it)]
+            idx.extend(range(o, o + n))
+        if not idx:
+            return None
+        sel = torch.tensor(idx, dtype=torch.long, device=wanted.device)
+        return wanted.index_select(0, sel).float()
 
     def execute(self, sched: SchedulerOutput) -> ExecuteResult:
         """Rank-0 entry point for one engine step (synchronous)."""

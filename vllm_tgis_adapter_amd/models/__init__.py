@@ -18,4 +18,8 @@ def get_model(cfg: ModelConfig):
         from .opt import OPTForCausalLM
 
         return OPTForCausalLM(cfg)
+    if cfg.architecture == "dolodra":
+        from .dolodra import DolodraForCausalLM
+
+        return DolodraForCausalLM(cfg)
     raise ValueError(f"Unsupported architecture: {cfg.architecture}")

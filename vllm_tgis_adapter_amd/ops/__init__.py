@@ -199,7 +199,7 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = No
     if (
         bias is None
         and x.dim() == 2
-        and _native(x)
+        and native_enabled(x)
         and x.dtype == torch.bfloat16
         and weight.dtype == torch.bfloat16
         and weight.shape[0] % 128 == 0
@@ -403,3 +403,173 @@ def topk_softmax(gate_logits: torch.Tensor, top_k: int):
 
 
 make_cos_sin_cache = reference.make_cos_sin_cache
+
+
+# ---------------------------------------------------------------------------
+# `_C_seq`: f32 residual-stream ops, short causal convolution with
+# per-sequence state, windowed latent attention with sinks.  A separate
+# extension so a model that needs only these compiles only these.
+# ---------------------------------------------------------------------------
+
+_S = None
+_seq_load_error: str | None = None
+
+
+def _try_load_seq() -> None:
+    global _S, _seq_load_error
+    if _S is not None:
+        return
+    try:
+        from vllm_tgis_adapter_amd import _C_seq as ext
+
+        _S = ext
+    except ImportError as e:
+        _seq_load_error = str(e)
+
+
+_try_load_seq()
+
+
+def has_native_seq() -> bool:
+    _try_load_seq()
+    return _S is not None
+
+
+def _native_seq(t: torch.Tensor) -> bool:
+    if t.device.type != "cuda" or _FORCE_REFERENCE:
+        return False
+    if _S is None:
+        _try_load_seq()
+    if _S is None:
+        raise RuntimeError(
+            "vllm_tgis_adapter_amd._C_seq HIP extension is not built but a GPU "
+            f"tensor reached one of its ops (import error: {_seq_load_error}). "
+            "Run `python kernels/build.py --only=_C_seq` first."
+        )
+    return True
+
+
+def gelu_tanh(x: torch.Tensor, mul: torch.Tensor | None = None) -> torch.Tensor:
+    """tanh-form GELU, optionally times ``mul`` (rows may be strided)."""
+    if x.numel() and _native_seq(x):
+        out = torch.empty_like(x)
+        _S.gelu_tanh(out, x, mul)
+        return out
+    return reference.gelu_tanh(x, mul)
+
+
+def embedding_scaled(ids: torch.Tensor, table: torch.Tensor, scale: float) -> torch.Tensor:
+    """f32 rows table[ids] * scale — the start of an f32 residual stream."""
+    if ids.numel() and _native_seq(table):
+        out = torch.empty((ids.shape[0], table.shape[1]), dtype=torch.float32,
+                          device=table.device)
+        _S.embedding_scaled(out, ids, table, float(scale))
+        return out
+    return reference.embedding_scaled(ids, table, scale)
+
+
+def rms_norm_stream(x: torch.Tensor, weight: torch.Tensor, eps: float,
+                    weight_offset: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """RMS norm of an f32 stream, weight applied as (weight_offset + w)."""
+    if x.numel() and _native_seq(x):
+        out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+        _S.rms_norm_stream(out, x, weight, float(eps), float(weight_offset))
+        return out
+    return reference.rms_norm_stream(x, weight, eps, weight_offset, out_dtype)
+
+
+def stream_add(x: torch.Tensor, a: torch.Tensor, b: torch.Tensor | None,
+               mult: float, cast_dtype: torch.dtype | None = None):
+    """x (f32, in place) += mult * (a + b); optionally also returns the new x
+    rounded to ``cast_dtype`` for the next projection."""
+    if x.numel() and _native_seq(x):
+        cast = (torch.empty(x.shape, dtype=cast_dtype, device=x.device)
+                if cast_dtype is not None else None)
+        _S.stream_add(x, a, b, float(mult), cast)
+        return cast
+    return reference.stream_add(x, a, b, mult, cast_dtype)
+
+
+def stream_add_rms_norm(x: torch.Tensor, y: torch.Tensor, weight: torch.Tensor,
+                        eps: float, mult: float) -> None:
+    """x (f32, in place) += mult * y / rms(y) * weight."""
+    if x.numel() and _native_seq(x):
+        _S.stream_add_rms_norm(x, y, weight, float(eps), float(mult))
+        return
+    reference.stream_add_rms_norm(x, y, weight, eps, mult)
+
+
+def softcap(logits: torch.Tensor, cap: float) -> torch.Tensor:
+    """f32 cap * tanh(logits / cap)."""
+    if logits.numel() and _native_seq(logits):
+        out = torch.empty(logits.shape, dtype=torch.float32, device=logits.device)
+        _S.softcap(out, logits.contiguous(), float(cap))
+        return out
+    return reference.softcap(logits, cap)
+
+
+def causal_conv_state(h, weight, state, seq_start_loc, seq_lens, state_slots,
+                      add_input: bool = True) -> torch.Tensor:
+    """Depthwise causal convolution over each sequence's new rows with the
+    last taps-1 inputs carried in ``state[slot]`` (advanced in place)."""
+    if h.numel() and _native_seq(h):
+        out = torch.empty_like(h)
+        _S.causal_conv_state(out, h, weight, state, seq_start_loc, seq_lens,
+                             state_slots, bool(add_input))
+        return out
+    return reference.causal_conv_state(
+        h, weight, state, seq_start_loc.cpu(), seq_lens.cpu(), state_slots.cpu(),
+        add_input)
+
+
+def rope_partial(x: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor,
+                 offset: int, rot_dims: int) -> None:
+    """In place half-split rotation of dims [offset, offset+rot_dims) of every
+    head of x [T, H, D]; f32 angles position * inv_freq[i]."""
+    if x.numel() and _native_seq(x):
+        _S.rope_partial(x, positions, inv_freq, int(offset), int(rot_dims))
+        return
+    reference.rope_partial(x, positions, inv_freq, offset, rot_dims)
+
+
+def latent_kv_write(dkv, norm_weight, eps, positions, inv_freq, rot_dims,
+                    cache, slot_mapping) -> None:
+    """RMS-norm the latent part, rotate the shared key part, store the row in
+    the paged latent cache."""
+    if dkv.numel() and _native_seq(dkv):
+        _S.latent_kv_write(dkv, norm_weight, float(eps), positions, inv_freq,
+                           int(rot_dims), cache, slot_mapping)
+        return
+    reference.latent_kv_write(dkv, norm_weight, eps, positions, inv_freq,
+                              rot_dims, cache, slot_mapping)
+
+
+def latent_attention_prefill(q_lat, q_rot, cache, block_tables, query_start_loc,
+                             seq_lens, scale, window, sinks, max_query_len,
+                             out: torch.Tensor) -> torch.Tensor:
+    """Windowed multi-query attention with sinks over the paged latent cache
+    for query chunks (the tail rows of each sequence)."""
+    if q_lat.numel() and _native_seq(q_lat):
+        _S.latent_attention_prefill(out, q_lat, q_rot, cache, block_tables,
+                                    query_start_loc, seq_lens, float(scale),
+                                    int(window), sinks, int(max_query_len), False)
+        return out
+    out.copy_(reference.latent_attention(
+        q_lat, q_rot, cache, block_tables.cpu(), query_start_loc.cpu(),
+        seq_lens.cpu(), scale, window, sinks))
+    return out
+
+
+def latent_attention_decode(q_lat, q_rot, cache, block_tables, seq_lens, scale,
+                            window, sinks, out: torch.Tensor) -> torch.Tensor:
+    """Same attention for one new query per sequence."""
+    if q_lat.numel() and _native_seq(q_lat):
+        _S.latent_attention_decode(out, q_lat, q_rot, cache, block_tables,
+                                   seq_lens, float(scale), int(window), sinks)
+        return out
+    n = q_lat.shape[0]
+    qsl = torch.arange(n + 1, dtype=torch.int32)
+    out.copy_(reference.latent_attention(
+        q_lat, q_rot, cache, block_tables.cpu(), qsl, seq_lens.cpu(), scale,
+        window, sinks))
+    return out
