@@ -39,13 +39,12 @@ void launch_latent_attention(T*, long, long, const T*, long, long, const T*,
                              const int*, int, const float*, float, int, int,
                              int, int, int, int, hipStream_t);
 bool latent_prefill_mfma_usable(int rank, int rot, int block_size);
-void launch_latent_prefill_mfma(__hip_bfloat16*, long, long,
-                                const __hip_bfloat16*, long, long,
-                                const __hip_bfloat16*, long, long,
-                                const __hip_bfloat16*, const int*, int,
-                                const int*, const int*, int, const float*,
-                                float, int, int, int, int, int, int,
-                                hipStream_t);
+void launch_latent_attn_mfma(__hip_bfloat16*, long, long,
+                             const __hip_bfloat16*, long, long,
+                             const __hip_bfloat16*, long, long,
+                             const __hip_bfloat16*, const int*, int, const int*,
+                             const int*, int, const float*, float, int, int,
+                             int, int, int, int, hipStream_t);
 
 namespace {
 
@@ -254,7 +253,7 @@ void latent_attention_common(torch::Tensor& out, torch::Tensor& q_lat,
                              torch::Tensor& seq_lens, double scale,
                              int64_t window,
                              c10::optional<torch::Tensor>& sinks,
-                             bool allow_mfma) {
+                             int max_q, bool allow_mfma) {
   TORCH_CHECK(q_lat.is_cuda() && q_lat.dim() == 3 && q_rot.dim() == 3 &&
               out.dim() == 3);
   TORCH_CHECK(q_lat.stride(2) == 1 && q_rot.stride(2) == 1 && out.stride(2) == 1);
@@ -282,15 +281,20 @@ void latent_attention_common(torch::Tensor& out, torch::Tensor& q_lat,
     sk = ptr<float>(sinks.value());
   }
   const int block_size = cache.size(1);
+  auto vec_ok = [](const torch::Tensor& t, int elems) {
+    return t.stride(0) % elems == 0 && t.stride(1) % elems == 0 &&
+           reinterpret_cast<uintptr_t>(t.data_ptr()) % (2 * elems) == 0;
+  };
   if (allow_mfma && q_lat.scalar_type() == at::ScalarType::BFloat16 &&
-      latent_prefill_mfma_usable(rank, rot, block_size)) {
+      latent_prefill_mfma_usable(rank, rot, block_size) && vec_ok(q_lat, 8) &&
+      vec_ok(q_rot, 8) && vec_ok(out, 4)) {
     using bf = __hip_bfloat16;
-    launch_latent_prefill_mfma(
+    launch_latent_attn_mfma(
         ptr<bf>(out), out.stride(0), out.stride(1), ptr<bf>(q_lat),
         q_lat.stride(0), q_lat.stride(1), ptr<bf>(q_rot), q_rot.stride(0),
         q_rot.stride(1), ptr<bf>(cache), ptr<int>(block_tables),
         (int)block_tables.stride(0), qsl, ptr<int>(seq_lens), nseq, sk,
-        (float)scale, (int)window, rows, heads, rank, rot, block_size, stream());
+        (float)scale, (int)window, max_q, heads, rank, rot, block_size, stream());
     return;
   }
   DISPATCH_F32_BF16(q_lat.scalar_type(), {
@@ -311,18 +315,19 @@ void latent_attention_prefill(torch::Tensor out, torch::Tensor q_lat,
                               int64_t max_query_len, bool generic) {
   check_i32(qsl, "query_start_loc");
   TORCH_CHECK(qsl.numel() == seq_lens.numel() + 1);
-  (void)max_query_len;
+  TORCH_CHECK(max_query_len >= 1, "max_query_len");
   latent_attention_common(out, q_lat, q_rot, cache, block_tables, ptr<int>(qsl),
-                          seq_lens, scale, window, sinks, !generic);
+                          seq_lens, scale, window, sinks, (int)max_query_len,
+                          !generic);
 }
 
 void latent_attention_decode(torch::Tensor out, torch::Tensor q_lat,
                              torch::Tensor q_rot, torch::Tensor cache,
                              torch::Tensor block_tables, torch::Tensor seq_lens,
                              double scale, int64_t window,
-                             c10::optional<torch::Tensor> sinks) {
+                             c10::optional<torch::Tensor> sinks, bool generic) {
   latent_attention_common(out, q_lat, q_rot, cache, block_tables, nullptr,
-                          seq_lens, scale, window, sinks, false);
+                          seq_lens, scale, window, sinks, 1, !generic);
 }
 
 }  // namespace

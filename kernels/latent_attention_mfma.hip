@@ -1,17 +1,269 @@
-// MFMA prompt-portion kernel for latent attention (bf16).  Placeholder until
-// the tiled kernel lands: reports "not usable", so the general kernel runs.
+// MFMA kernel for windowed latent attention with sinks (bf16 storage).
+//
+// All heads of a token score the SAME cached row [rank + rot] and sum the same
+// latent, so the natural matrix shape is: rows = (token, head) pairs, columns =
+// keys.  One workgroup (4 waves) owns 64 such rows — 64/H consecutive tokens of
+// one sequence times its H heads (or one token and 64 heads of it when H > 64)
+// — and walks the keys its tokens can see in tiles of 32.  A single decoding
+// token is the case "one token per workgroup".
+//
+// Per tile:
+//   stage   the 32 rows are copied once into LDS (K image, padded rows) and
+//           their latent part once more transposed (V^T image) — every wave
+//           and every head reuses both
+//   scores  swapped operands, S^T = K . Q^T on v_mfma_f32_16x16x32_bf16: a lane
+//           then holds 8 scores of ONE query row, so max and sum need two
+//           xor-shuffles, and the bf16 probabilities are already laid out as
+//           the B operand of the next product (the key order inside the
+//           contraction is permuted to match; the V^T image is stored in that
+//           same slot order so its A fragments are single 16-byte reads)
+//   values  O^T += V^T . P^T, rank/16 accumulator tiles per wave, rescaled by
+//           the per-row online-softmax factor
+// Scores, softmax statistics and accumulators are f32; the sink enters the
+// denominator at the end.  Window and causality are applied per element from
+// the row's position.  Shapes are compile-time (rank/16, (rank+rot)/32) for a
+// fixed list; other shapes use the general kernel.
 
 #include "common.h"
 
+typedef __attribute__((ext_vector_type(8))) short bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+typedef __hip_bfloat16 bf16;
+
+#define LM_THREADS 256
+#define LM_ROWS 64
+#define LM_KT 32
+#define LM_KPAD 8
+#define LM_VROW 40
+
+DEVINLINE short f32_to_bf16_bits(float x) {
+  return __builtin_bit_cast(short, __float2bfloat16(x));
+}
+
+template <int NT, int KS>
+__global__ __launch_bounds__(LM_THREADS) void latent_attn_mfma_kernel(
+    bf16* __restrict__ out, long o_st, long o_sh,
+    const bf16* __restrict__ q_lat, long ql_st, long ql_sh,
+    const bf16* __restrict__ q_rot, long qr_st, long qr_sh,
+    const bf16* __restrict__ cache, const int* __restrict__ block_tables,
+    int bt_stride, const int* __restrict__ qsl, const int* __restrict__ seq_lens,
+    const float* __restrict__ sinks, float scale, int window, int heads, int tq,
+    int hpb, int block_size) {
+  constexpr int RANK = NT * 16;
+  constexpr int D = KS * 32;
+  constexpr int KROW = D + LM_KPAD;
+  extern __shared__ char lds_raw[];
+  bf16* k_img = reinterpret_cast<bf16*>(lds_raw);   // [32][KROW]
+  bf16* v_img = k_img + LM_KT * KROW;               // [RANK][LM_VROW]
+
+  const int seq = blockIdx.y;
+  int q0, nq;
+  if (qsl != nullptr) {
+    q0 = qsl[seq];
+    nq = qsl[seq + 1] - q0;
+  } else {
+    q0 = seq;
+    nq = 1;
+  }
+  const int slen = seq_lens[seq];
+  const int t0 = blockIdx.x * tq;
+  if (t0 >= nq) return;
+  const int nt = min(tq, nq - t0);
+  const int h0 = blockIdx.z * hpb;
+  const int nh = min(hpb, heads - h0);
+  const int nrows = nt * nh;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n = lane & 15, g = lane >> 4;
+  const int r = wave * 16 + n;
+  const bool row_ok = r < nrows;
+  const int tl = row_ok ? r / nh : 0;
+  const int head = h0 + (row_ok ? r % nh : 0);
+  const long qrow = q0 + t0 + tl;
+  bf16* orow = out + qrow * o_st + head * o_sh;
+
+  if (slen <= 0) {   // padding row of a captured bucket
+    if (row_ok)
+      for (int k = g; k < RANK; k += 4) orow[k] = __float2bfloat16(0.f);
+    return;
+  }
+
+  const int pos0 = slen - nq + t0;
+  const int kend = pos0 + nt;
+  const int kstart = (window > 0) ? max(0, pos0 - window + 1) : 0;
+  const int qpos = pos0 + tl;
+  const int klo = (window > 0) ? qpos - window + 1 : 0;
+  const int* bt = block_tables + (long)seq * bt_stride;
+  const bool wave_active = wave * 16 < nrows;
+
+  bf16x8_t qf[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    const int dim = ks * 32 + g * 8;
+    bf16x8_t v = {};
+    if (row_ok) {
+      const bf16* src = (dim < RANK)
+          ? q_lat + qrow * ql_st + head * ql_sh + dim
+          : q_rot + qrow * qr_st + head * qr_sh + (dim - RANK);
+      v = *reinterpret_cast<const bf16x8_t*>(src);
+    }
+    qf[ks] = v;
+  }
+
+  f32x4_t acc[NT];
+#pragma unroll
+  for (int i = 0; i < NT; ++i) acc[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  float m_run = -INFINITY, l_part = 0.f;
+
+  for (int base = kstart; base < kend; base += LM_KT) {
+    __syncthreads();   // readers of the previous tile's images are done
+    for (int c = tid; c < LM_KT * (D / 8); c += LM_THREADS) {
+      const int key = c / (D / 8), ch = c - key * (D / 8);
+      const int kk = min(base + key, kend - 1);
+      const long off = ((long)bt[kk / block_size] * block_size + (kk % block_size)) * D + ch * 8;
+      *reinterpret_cast<bf16x8_t*>(k_img + key * KROW + ch * 8) =
+          *reinterpret_cast<const bf16x8_t*>(cache + off);
+    }
+    __syncthreads();
+    // latent part once more, transposed, keys in contraction-slot order
+    for (int c = tid; c < LM_KT * (RANK / 8); c += LM_THREADS) {
+      const int key = c & 31, ch = c >> 5;
+      const bf16x8_t v = *reinterpret_cast<const bf16x8_t*>(k_img + key * KROW + ch * 8);
+      const int slot = ((key & 15) >> 2) * 8 + (key >> 4) * 4 + (key & 3);
+      short* dst = reinterpret_cast<short*>(v_img) + (ch * 8) * LM_VROW + slot;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) dst[u * LM_VROW] = v[u];
+    }
+
+    f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+    if (wave_active) {
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const bf16x8_t a0 = *reinterpret_cast<const bf16x8_t*>(
+            k_img + n * KROW + ks * 32 + g * 8);
+        const bf16x8_t a1 = *reinterpret_cast<const bf16x8_t*>(
+            k_img + (16 + n) * KROW + ks * 32 + g * 8);
+        s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, qf[ks], s0, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, qf[ks], s1, 0, 0, 0);
+      }
+    }
+    float sv[8];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int kk = base + (i >> 2) * 16 + 4 * g + (i & 3);
+      const bool ok = row_ok && kk <= qpos && kk >= klo;
+      const float s = (i < 4 ? s0[i & 3] : s1[i & 3]) * scale;
+      sv[i] = ok ? s : -INFINITY;
+      mx = fmaxf(mx, sv[i]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE_SIZE));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE_SIZE));
+    const float m_new = fmaxf(m_run, mx);
+    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+    const float alpha = (m_run == -INFINITY) ? 0.f : __expf(m_run - m_safe);
+    bf16x8_t pb;
+    float ps = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float p = (sv[i] == -INFINITY) ? 0.f : __expf(sv[i] - m_safe);
+      ps += p;
+      pb[i] = f32_to_bf16_bits(p);
+    }
+    l_part = l_part * alpha + ps;
+    m_run = m_new;
+#pragma unroll
+    for (int i = 0; i < NT; ++i) {
+      acc[i][0] *= alpha; acc[i][1] *= alpha; acc[i][2] *= alpha; acc[i][3] *= alpha;
+    }
+    __syncthreads();   // V^T image complete
+    if (wave_active) {
+#pragma unroll
+      for (int dt = 0; dt < NT; ++dt) {
+        const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(
+            v_img + (dt * 16 + n) * LM_VROW + g * 8);
+        acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb, acc[dt], 0, 0, 0);
+      }
+    }
+  }
+
+  float l = l_part;
+  l += __shfl_xor(l, 16, WAVE_SIZE);
+  l += __shfl_xor(l, 32, WAVE_SIZE);
+  float rescale = 1.f;
+  if (sinks != nullptr) {
+    const float sk = sinks[head];
+    const float m_fin = fmaxf(m_run, sk);
+    rescale = (m_run == -INFINITY) ? 0.f : __expf(m_run - m_fin);
+    l = l * rescale + __expf(sk - m_fin);
+  }
+  const float inv = (l > 0.f) ? rescale / l : 0.f;
+  if (row_ok) {
+#pragma unroll
+    for (int dt = 0; dt < NT; ++dt) {
+      union { short s[4]; uint2 v; } o;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o.s[i] = f32_to_bf16_bits(acc[dt][i] * inv);
+      *reinterpret_cast<uint2*>(orow + dt * 16 + 4 * g) = o.v;
+    }
+  }
+}
+
+#define LM_SHAPES(X) \
+  X(2, 2) X(2, 3) X(4, 3) X(4, 4) X(6, 4) X(6, 5) X(8, 5) X(8, 6) X(16, 9) \
+  X(16, 10) X(32, 17) X(32, 18)
+
 bool latent_prefill_mfma_usable(int rank, int rot, int block_size) {
-  (void)rank; (void)rot; (void)block_size;
+  (void)block_size;
+  if (rank % 16 != 0 || (rank + rot) % 32 != 0 || rot % 8 != 0) return false;
+  const int nt = rank / 16, ks = (rank + rot) / 32;
+#define X(A, B) if (nt == A && ks == B) return true;
+  LM_SHAPES(X)
+#undef X
   return false;
 }
 
-void launch_latent_prefill_mfma(__hip_bfloat16*, long, long,
-                                const __hip_bfloat16*, long, long,
-                                const __hip_bfloat16*, long, long,
-                                const __hip_bfloat16*, const int*, int,
-                                const int*, const int*, int, const float*,
-                                float, int, int, int, int, int, int,
-                                hipStream_t) {}
+template <int NT, int KS>
+static void launch_one(bf16* out, long o_st, long o_sh, const bf16* q_lat,
+                       long ql_st, long ql_sh, const bf16* q_rot, long qr_st,
+                       long qr_sh, const bf16* cache, const int* block_tables,
+                       int bt_stride, const int* qsl, const int* seq_lens,
+                       int nseq, const float* sinks, float scale, int window,
+                       int max_q, int heads, int block_size, hipStream_t stream) {
+  constexpr int RANK = NT * 16, D = KS * 32;
+  const size_t smem = sizeof(bf16) * (LM_KT * (D + LM_KPAD) + RANK * LM_VROW);
+  static bool configured = false;
+  if (!configured) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&latent_attn_mfma_kernel<NT, KS>),
+                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    configured = true;
+  }
+  const int hpb = heads < LM_ROWS ? heads : LM_ROWS;
+  const int tq = LM_ROWS / hpb;
+  dim3 grid((max_q + tq - 1) / tq, nseq, (heads + hpb - 1) / hpb);
+  latent_attn_mfma_kernel<NT, KS><<<grid, LM_THREADS, smem, stream>>>(
+      out, o_st, o_sh, q_lat, ql_st, ql_sh, q_rot, qr_st, qr_sh, cache,
+      block_tables, bt_stride, qsl, seq_lens, sinks, scale, window, heads, tq,
+      hpb, block_size);
+}
+
+void launch_latent_attn_mfma(bf16* out, long o_st, long o_sh, const bf16* q_lat,
+                             long ql_st, long ql_sh, const bf16* q_rot,
+                             long qr_st, long qr_sh, const bf16* cache,
+                             const int* block_tables, int bt_stride,
+                             const int* qsl, const int* seq_lens, int nseq,
+                             const float* sinks, float scale, int window,
+                             int max_q, int heads, int rank, int rot,
+                             int block_size, hipStream_t stream) {
+  const int nt = rank / 16, ks = (rank + rot) / 32;
+#define X(A, B)                                                               \
+  if (nt == A && ks == B) {                                                   \
+    launch_one<A, B>(out, o_st, o_sh, q_lat, ql_st, ql_sh, q_rot, qr_st,     \
+                     qr_sh, cache, block_tables, bt_stride, qsl, seq_lens,    \
+                     nseq, sinks, scale, window, max_q, heads, block_size,    \
+                     stream);                                                 \
+    return;                                                                   \
+  }
+  LM_SHAPES(X)
+#undef X
+}

@@ -156,3 +156,49 @@ def test_latent_attention(dtype, rank, rot, window):
         q_lat[rows], q_rot[rows], cache, tables,
         torch.arange(len(seqs) + 1, dtype=torch.int32), lens, scale, window, None)
     torch.testing.assert_close(out_d.cpu().float(), want_d.float(), **_tol(dtype))
+
+
+@pytest.mark.parametrize("rank,rot,heads,window,bs", [
+    (32, 32, 3, 5, 4), (64, 32, 4, 40, 16), (96, 32, 6, 21, 8), (96, 64, 16, 0, 16),
+    (128, 64, 70, 33, 8), (256, 32, 16, 100, 16), (512, 64, 16, 64, 16), (512, 32, 5, 0, 32),
+])
+def test_latent_attention_mfma(rank, rot, heads, window, bs):
+    """The bf16 MFMA kernel (prompt portions and single queries) against the
+    f32 reference and against the general kernel."""
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(rank + heads)
+    nb = 40 * 16 // bs + 8
+    cache = torch.randn(nb, bs, rank + rot, generator=g).to(dtype)
+    seqs = [(3, 3), (200, 70), (65, 1), (33, 2), (130, 130 if window == 0 else 45)]
+    tables = torch.zeros(len(seqs), nb, dtype=torch.int32)
+    for i, (ctx, _) in enumerate(seqs):
+        n = (ctx + bs - 1) // bs
+        tables[i, :n] = torch.randperm(nb, generator=g)[:n].to(torch.int32)
+    qsl = torch.tensor([0] + list(torch.tensor([n for _, n in seqs]).cumsum(0)), dtype=torch.int32)
+    lens = torch.tensor([c for c, _ in seqs], dtype=torch.int32)
+    t = int(qsl[-1])
+    scale = 2.0 / (rank + rot) ** 0.5
+    q_lat = torch.randn(heads, t, rank, generator=g).to(dtype).transpose(0, 1)
+    q_full = torch.randn(t, heads, 8 + rot, generator=g).to(dtype)
+    q_rot = q_full[:, :, 8:]
+    sinks = torch.randn(heads, generator=g)
+    want = ref.latent_attention(q_lat.float(), q_rot.float(), cache.float(), tables, qsl, lens,
+                                scale, window, sinks)
+    args = (q_lat.cuda(), q_rot.cuda(), cache.cuda(), tables.cuda(), qsl.cuda(), lens.cuda(),
+            scale, window, sinks.cuda(), max(n for _, n in seqs))
+    out = torch.full((heads, t, rank), float("nan"), dtype=dtype, device="cuda").transpose(0, 1)
+    ops.latent_attention_prefill(*args, out=out)
+    gen = torch.empty(heads, t, rank, dtype=dtype, device="cuda").transpose(0, 1)
+    ops.latent_attention_prefill(*args, out=gen, general=True)
+    torch.testing.assert_close(out.cpu().float(), want, atol=3e-2, rtol=3e-2)
+    torch.testing.assert_close(out.cpu().float(), gen.cpu().float(), atol=3e-2, rtol=3e-2)
+
+    rows = (qsl[1:] - 1).long()
+    out_d = torch.full((len(seqs), heads, rank), float("nan"), dtype=dtype, device="cuda")
+    ops.latent_attention_decode(
+        q_lat[rows].contiguous().cuda(), q_rot[rows].cuda(), cache.cuda(), tables.cuda(),
+        lens.cuda(), scale, window, sinks.cuda(), out=out_d)
+    want_d = ref.latent_attention(
+        q_lat[rows].float(), q_rot[rows].float(), cache.float(), tables,
+        torch.arange(len(seqs) + 1, dtype=torch.int32), lens, scale, window, sinks)
+    torch.testing.assert_close(out_d.cpu().float(), want_d, atol=3e-2, rtol=3e-2)

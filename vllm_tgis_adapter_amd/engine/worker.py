@@ -637,8 +637,8 @@ class Worker:
             self.graph_runner is not None
             and np_seqs == 0
             and not batch.get("lora_ids")
-            and batch["num_sample_rows"] == n
             and len(batch["logit_rows"]) == n
+            and list(batch["logit_rows"]) == list(range(n))
             and self.graph_runner.bucket_for(n) is not None
         ):
             slots = self._h2d("slots", np.asarray(batch["slot_mapping"], dtype=np.int64), torch.int64)
