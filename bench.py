@@ -39,7 +39,13 @@ def parse_args():
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=32)
     p.add_argument("--warmup", type=int, default=8)
-    p.add_argument("--mode", choices=["serve", "engine"], default="serve")
+    p.add_argument("--mode", choices=["serve", "engine", "arch"], default="serve",
+                   help="arch: prefill/decode throughput of the Dolodra design "
+                        "beside a llama of equal size (engine loop, random weights)")
+    p.add_argument("--arch-sizes", type=str, default="s,m",
+                   help="arch mode: comma list of sizes (s, m)")
+    p.add_argument("--arch-models", type=str, default="dolodra,llama",
+                   help="arch mode: which of the two models to run")
     p.add_argument("--model", type=str, default="llama-3-8b")
     p.add_argument("--batch", type=int, default=512)
     p.add_argument("--prompt-len", type=int, default=512)
@@ -461,6 +467,131 @@ def run_engine(args, device: str) -> None:
     print(json.dumps(out))
 
 
+# ---------------------------------------------------------------------------
+# --mode arch: the Dolodra design beside the closest existing model (llama)
+# at equal width / depth / parameter count, random weights, through the same
+# engine loop (scheduler + forward + sampler).  Reports prefill tokens/s (all
+# prompts to their first token) and decode tokens/s (K steps of a full batch).
+# ---------------------------------------------------------------------------
+
+ARCH_SIZES = {
+    # ~1B-class layers: 16 heads, latent 256 + 32 rotated, window 512
+    "s": dict(width=2048, layers=8, vocab=32000, heads=16, dim=128, rot=32, vdim=128,
+              rank=256, window=512, ff=8448, llama_inter=5632, llama_kv_heads=4),
+    # ~8B-class layers: 32 heads, latent 512 + 64 rotated, window 1024
+    "m": dict(width=4096, layers=8, vocab=32000, heads=32, dim=128, rot=64, vdim=128,
+              rank=512, window=1024, ff=21504, llama_inter=14336, llama_kv_heads=8),
+    # CPU dry run
+    "t": dict(width=64, layers=2, vocab=512, heads=4, dim=16, rot=16, vdim=16,
+              rank=32, window=24, ff=192, llama_inter=128, llama_kv_heads=2),
+}
+
+
+def _arch_model_configs(sz: dict, dtype: str):
+    from vllm_tgis_adapter_amd.engine import ModelConfig
+    from vllm_tgis_adapter_amd.engine.config import _DTYPES
+    from vllm_tgis_adapter_amd.models.dolodra import model_config_from_json
+
+    layers = []
+    for i in range(sz["layers"]):
+        mixer = {"heads": sz["heads"], "dim": sz["dim"], "rot_dim": sz["rot"],
+                 "vdim": sz["vdim"], "kv_rank": sz["rank"],
+                 "scale": (sz["dim"] + sz["rot"]) ** -0.5, "mask": {"size": sz["window"]},
+                 "rot": {"base": 10000.0, "dims": sz["rot"]}}
+        if i % 2 == 1:
+            mixer["kv_from"] = i - 1   # every second layer borrows the latent
+        layers.append({"type": "latent_attention", "mixer": mixer,
+                       "mlp": {"kind": "dense", "ff": sz["ff"]}})
+    hf = {"architecture": "Dolodra", "vocab": sz["vocab"], "width": sz["width"],
+          "layers": layers, "norm": {"eps": 1e-5}, "residual_mult": 0.5,
+          "logit_softcap": 30.0, "embedding": {"scale": sz["width"] ** 0.5},
+          "canon": {"taps": 4}, "token_side": {"dim": 32}}
+    dolo = model_config_from_json("dolodra-synthetic", hf)
+    dolo.dtype = _DTYPES[dtype]
+    llama = ModelConfig(
+        model="llama-equal", architecture="llama", vocab_size=sz["vocab"],
+        hidden_size=sz["width"], intermediate_size=sz["llama_inter"],
+        num_layers=sz["layers"], num_heads=sz["heads"],
+        num_kv_heads=sz["llama_kv_heads"], head_dim=sz["width"] // sz["heads"],
+        rope_theta=500000.0, rms_norm_eps=1e-5, max_model_len=8192,
+        tie_word_embeddings=False, dtype=_DTYPES[dtype])
+    return dolo, llama
+
+
+def _arch_measure(mc, args, device: str, batch: int, prompt_len: int, steps: int,
+                  warmup: int) -> dict:
+    from vllm_tgis_adapter_amd.engine import EngineConfig, LLMEngine, SamplingParams
+    from vllm_tgis_adapter_amd.engine.config import CacheConfig, SchedulerConfig
+
+    bs = args.block_size
+    per_seq = (prompt_len + steps + warmup + 8 + bs - 1) // bs
+    cfg = EngineConfig(
+        model_config=mc,
+        cache_config=CacheConfig(block_size=bs, num_gpu_blocks=batch * per_seq + 16),
+        scheduler_config=SchedulerConfig(max_num_seqs=batch, max_num_batched_tokens=8192,
+                                         prefill_admit_batch=1),
+        device=device, enforce_eager=args.enforce_eager)
+    engine = LLMEngine(cfg)
+    sync = torch.cuda.synchronize if device == "cuda" else (lambda: None)
+    g = torch.Generator().manual_seed(0)
+    res = {}
+    for rnd in range(2):   # round 0 warms allocators / GEMM heuristics
+        for i in range(batch):
+            ids = torch.randint(4, mc.vocab_size, (prompt_len,), generator=g).tolist()
+            engine.add_request(f"r{rnd}-{i}", None, ids,
+                               SamplingParams(temperature=0.0, max_tokens=steps + warmup + 4,
+                                              min_tokens=steps + warmup + 4))
+        sync()
+        t0 = time.perf_counter()
+        while engine.scheduler.waiting or any(r.is_prefilling for r in engine.scheduler.running):
+            engine.step()
+        sync()
+        t1 = time.perf_counter()
+        for _ in range(warmup):
+            engine.step()
+        sync()
+        t2 = time.perf_counter()
+        for _ in range(steps):
+            engine.step()
+        sync()
+        t3 = time.perf_counter()
+        res = {"prefill_tok_s": batch * prompt_len / (t1 - t0),
+               "decode_tok_s": batch * steps / (t3 - t2),
+               "decode_ms_per_step": (t3 - t2) / steps * 1e3}
+        for rid in [r.request_id for r in list(engine.scheduler.running)]:
+            engine.abort_request(rid)
+        while engine.has_unfinished():
+            engine.step()
+    del engine
+    if device == "cuda":
+        torch.cuda.empty_cache()
+    return res
+
+
+def run_arch(args, device: str) -> None:
+    out = []
+    sizes = ["t"] if device == "cpu" else args.arch_sizes.split(",")
+    for name in sizes:
+        sz = ARCH_SIZES[name]
+        dolo, llama = _arch_model_configs(sz, args.dtype)
+        batch = min(args.batch, 256) if device == "cuda" else 4
+        plen = args.prompt_len if device == "cuda" else 32
+        steps = args.steps if device == "cuda" else 4
+        warm = args.warmup if device == "cuda" else 1
+        for label, mc in (("dolodra", dolo), ("llama", llama)):
+            if label not in args.arch_models.split(","):
+                continue
+            r = _arch_measure(mc, args, device, batch, plen, steps, warm)
+            r.update(size=name, model=label, batch=batch, prompt_len=plen)
+            out.append(r)
+            print(f"[arch] size={name} {label:8s} batch={batch} prompt={plen}: "
+                  f"prefill {r['prefill_tok_s']:.0f} tok/s, decode {r['decode_tok_s']:.0f} tok/s "
+                  f"({r['decode_ms_per_step']:.2f} ms/step)", file=sys.stderr, flush=True)
+    print(json.dumps({"metric": "arch_compare_tokens_per_s", "unit": "tokens/s",
+                      "dtype": args.dtype, "data": "synthetic", "steps": args.steps,
+                      "warmup": args.warmup, "results": out}))
+
+
 def main():
     args = parse_args()
     world = int(os.environ.get("WORLD_SIZE", str(args.gpus)))
@@ -474,7 +605,9 @@ def main():
         args.batch = min(args.batch, 64)
         args.prompt_len = min(args.prompt_len, 64)
 
-    if args.mode == "serve":
+    if args.mode == "arch":
+        run_arch(args, device)
+    elif args.mode == "serve":
         run_serve(args, device)
     else:
         run_engine(args, device)

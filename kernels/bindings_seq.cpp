@@ -44,7 +44,9 @@ void launch_latent_attn_mfma(__hip_bfloat16*, long, long,
                              const __hip_bfloat16*, long, long,
                              const __hip_bfloat16*, const int*, int, const int*,
                              const int*, int, const float*, float, int, int,
-                             int, int, int, int, hipStream_t);
+                             int, int, int, int, int, float*, float*,
+                             hipStream_t);
+int latent_decode_num_splits(int nseq, int heads, int max_keys);
 
 namespace {
 
@@ -289,12 +291,27 @@ void latent_attention_common(torch::Tensor& out, torch::Tensor& q_lat,
       latent_prefill_mfma_usable(rank, rot, block_size) && vec_ok(q_lat, 8) &&
       vec_ok(q_rot, 8) && vec_ok(out, 4)) {
     using bf = __hip_bfloat16;
+    // single-query steps: slice the keys over workgroups (shape-pure count)
+    int nsplit = 1;
+    torch::Tensor part_acc, part_ml;
+    if (qsl == nullptr) {
+      const int max_keys = window > 0
+          ? (int)window : (int)(block_tables.size(1) * block_size);
+      nsplit = latent_decode_num_splits(nseq, heads, max_keys);
+      if (nsplit > 1) {
+        auto opt = torch::TensorOptions().dtype(torch::kFloat32).device(out.device());
+        part_acc = torch::empty({(long)nseq * nsplit * heads * rank}, opt);
+        part_ml = torch::empty({(long)nseq * nsplit * heads * 2}, opt);
+      }
+    }
     launch_latent_attn_mfma(
         ptr<bf>(out), out.stride(0), out.stride(1), ptr<bf>(q_lat),
         q_lat.stride(0), q_lat.stride(1), ptr<bf>(q_rot), q_rot.stride(0),
         q_rot.stride(1), ptr<bf>(cache), ptr<int>(block_tables),
         (int)block_tables.stride(0), qsl, ptr<int>(seq_lens), nseq, sk,
-        (float)scale, (int)window, max_q, heads, rank, rot, block_size, stream());
+        (float)scale, (int)window, max_q, heads, rank, rot, block_size, nsplit,
+        nsplit > 1 ? ptr<float>(part_acc) : nullptr,
+        nsplit > 1 ? ptr<float>(part_ml) : nullptr, stream());
     return;
   }
   DISPATCH_F32_BF16(q_lat.scalar_type(), {

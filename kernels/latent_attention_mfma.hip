@@ -48,7 +48,8 @@ __global__ __launch_bounds__(LM_THREADS) void latent_attn_mfma_kernel(
     const bf16* __restrict__ cache, const int* __restrict__ block_tables,
     int bt_stride, const int* __restrict__ qsl, const int* __restrict__ seq_lens,
     const float* __restrict__ sinks, float scale, int window, int heads, int tq,
-    int hpb, int block_size) {
+    int hpb, int block_size, int nsplit, float* __restrict__ part_acc,
+    float* __restrict__ part_ml) {
   constexpr int RANK = NT * 16;
   constexpr int D = KS * 32;
   constexpr int KROW = D + LM_KPAD;
@@ -66,7 +67,9 @@ __global__ __launch_bounds__(LM_THREADS) void latent_attn_mfma_kernel(
     nq = 1;
   }
   const int slen = seq_lens[seq];
-  const int t0 = blockIdx.x * tq;
+  // nsplit > 1 (single-query steps only): blockIdx.x is a slice of the keys
+  const int split = (nsplit > 1) ? blockIdx.x : 0;
+  const int t0 = (nsplit > 1) ? 0 : blockIdx.x * tq;
   if (t0 >= nq) return;
   const int nt = min(tq, nq - t0);
   const int h0 = blockIdx.z * hpb;
@@ -83,14 +86,24 @@ __global__ __launch_bounds__(LM_THREADS) void latent_attn_mfma_kernel(
   bf16* orow = out + qrow * o_st + head * o_sh;
 
   if (slen <= 0) {   // padding row of a captured bucket
-    if (row_ok)
+    if (row_ok && split == 0)
       for (int k = g; k < RANK; k += 4) orow[k] = __float2bfloat16(0.f);
+    if (nsplit > 1 && row_ok && g == 0) {
+      float* ml = part_ml + (((long)seq * nsplit + split) * heads + head) * 2;
+      ml[0] = -INFINITY;
+      ml[1] = -1.f;     // tells the merge: nothing to do, the row is zero already
+    }
     return;
   }
 
   const int pos0 = slen - nq + t0;
-  const int kend = pos0 + nt;
-  const int kstart = (window > 0) ? max(0, pos0 - window + 1) : 0;
+  int kend = pos0 + nt;
+  int kstart = (window > 0) ? max(0, pos0 - window + 1) : 0;
+  if (nsplit > 1) {
+    const int per = ((kend - kstart + nsplit - 1) / nsplit + LM_KT - 1) / LM_KT * LM_KT;
+    kstart = kstart + split * per;
+    kend = min(kend, kstart + per);
+  }
   const int qpos = pos0 + tl;
   const int klo = (window > 0) ? qpos - window + 1 : 0;
   const int* bt = block_tables + (long)seq * bt_stride;
@@ -115,15 +128,36 @@ __global__ __launch_bounds__(LM_THREADS) void latent_attn_mfma_kernel(
   for (int i = 0; i < NT; ++i) acc[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   float m_run = -INFINITY, l_part = 0.f;
 
+  // global loads of a tile are issued one tile ahead and parked in registers:
+  // their latency hides under the previous tile's products
+  constexpr int CPR = D / 8;                                     // 16-byte chunks per row
+  constexpr int CPT = (LM_KT * CPR + LM_THREADS - 1) / LM_THREADS;  // chunks per thread
+  bf16x8_t pre[CPT];
+  auto fetch = [&](int base) {
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) {
+      const int c = tid + i * LM_THREADS;
+      if (c < LM_KT * CPR) {
+        const int key = c / CPR, ch = c - key * CPR;
+        const int kk = min(base + key, kend - 1);
+        const long off = ((long)bt[kk / block_size] * block_size + (kk % block_size)) * D + ch * 8;
+        pre[i] = *reinterpret_cast<const bf16x8_t*>(cache + off);
+      }
+    }
+  };
+  if (kstart < kend) fetch(kstart);
+
   for (int base = kstart; base < kend; base += LM_KT) {
     __syncthreads();   // readers of the previous tile's images are done
-    for (int c = tid; c < LM_KT * (D / 8); c += LM_THREADS) {
-      const int key = c / (D / 8), ch = c - key * (D / 8);
-      const int kk = min(base + key, kend - 1);
-      const long off = ((long)bt[kk / block_size] * block_size + (kk % block_size)) * D + ch * 8;
-      *reinterpret_cast<bf16x8_t*>(k_img + key * KROW + ch * 8) =
-          *reinterpret_cast<const bf16x8_t*>(cache + off);
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) {
+      const int c = tid + i * LM_THREADS;
+      if (c < LM_KT * CPR) {
+        const int key = c / CPR, ch = c - key * CPR;
+        *reinterpret_cast<bf16x8_t*>(k_img + key * KROW + ch * 8) = pre[i];
+      }
     }
+    if (base + LM_KT < kend) fetch(base + LM_KT);
     __syncthreads();
     // latent part once more, transposed, keys in contraction-slot order
     for (int c = tid; c < LM_KT * (RANK / 8); c += LM_THREADS) {
@@ -190,6 +224,20 @@ __global__ __launch_bounds__(LM_THREADS) void latent_attn_mfma_kernel(
   float l = l_part;
   l += __shfl_xor(l, 16, WAVE_SIZE);
   l += __shfl_xor(l, 32, WAVE_SIZE);
+  if (nsplit > 1) {
+    // unnormalised slice result; the merge kernel adds the sink and divides
+    if (row_ok) {
+      const long pr = ((long)seq * nsplit + split) * heads + head;
+      if (g == 0) {
+        part_ml[pr * 2] = m_run;
+        part_ml[pr * 2 + 1] = l;
+      }
+#pragma unroll
+      for (int dt = 0; dt < NT; ++dt)
+        *reinterpret_cast<f32x4_t*>(part_acc + pr * RANK + dt * 16 + 4 * g) = acc[dt];
+    }
+    return;
+  }
   float rescale = 1.f;
   if (sinks != nullptr) {
     const float sk = sinks[head];
@@ -207,6 +255,49 @@ __global__ __launch_bounds__(LM_THREADS) void latent_attn_mfma_kernel(
       *reinterpret_cast<uint2*>(orow + dt * 16 + 4 * g) = o.v;
     }
   }
+}
+
+// Sum of the key slices of a single-query step: out = sum_s acc_s e^(m_s - m)
+// / (sum_s l_s e^(m_s - m) + e^(sink - m)), m the max over slices and sink.
+__global__ void latent_attn_merge_kernel(bf16* __restrict__ out, long o_st, long o_sh,
+                                         const float* __restrict__ part_acc,
+                                         const float* __restrict__ part_ml,
+                                         const float* __restrict__ sinks,
+                                         int nsplit, int heads, int rank) {
+  const int seq = blockIdx.x, head = blockIdx.y;
+  const long p0 = ((long)seq * nsplit) * heads + head;
+  if (part_ml[p0 * 2 + 1] < 0.f) return;   // padding row, zeroed by the slices
+  float m = (sinks != nullptr) ? sinks[head] : -INFINITY;
+  for (int s = 0; s < nsplit; ++s) m = fmaxf(m, part_ml[(p0 + (long)s * heads) * 2]);
+  float l = (sinks != nullptr) ? __expf(sinks[head] - m) : 0.f;
+  for (int s = 0; s < nsplit; ++s) {
+    const float ms = part_ml[(p0 + (long)s * heads) * 2];
+    if (ms != -INFINITY) l += part_ml[(p0 + (long)s * heads) * 2 + 1] * __expf(ms - m);
+  }
+  const float inv = (l > 0.f) ? 1.f / l : 0.f;
+  bf16* orow = out + seq * o_st + head * o_sh;
+  for (int k = threadIdx.x; k < rank; k += blockDim.x) {
+    float a = 0.f;
+    for (int s = 0; s < nsplit; ++s) {
+      const long pr = p0 + (long)s * heads;
+      const float ms = part_ml[pr * 2];
+      if (ms != -INFINITY) a += part_acc[pr * rank + k] * __expf(ms - m);
+    }
+    orow[k] = __float2bfloat16(a * inv);
+  }
+}
+
+// Key slices per sequence for single-query steps: a pure function of shapes
+// (captured graphs replay the same grid).  Slices cost an f32 partial row per
+// (slice, head) written and read again, so they are only used to give every CU
+// a workgroup when the batch alone does not.
+int latent_decode_num_splits(int nseq, int heads, int max_keys) {
+  const int groups = (heads + LM_ROWS - 1) / LM_ROWS;
+  const int tiles = (max_keys + LM_KT - 1) / LM_KT;
+  int want = (256 + nseq * groups - 1) / (nseq * groups);
+  if (want > tiles / 2) want = tiles / 2;   // at least two tiles per slice
+  if (want > 32) want = 32;
+  return want < 1 ? 1 : want;
 }
 
 #define LM_SHAPES(X) \
@@ -229,7 +320,8 @@ static void launch_one(bf16* out, long o_st, long o_sh, const bf16* q_lat,
                        long qr_sh, const bf16* cache, const int* block_tables,
                        int bt_stride, const int* qsl, const int* seq_lens,
                        int nseq, const float* sinks, float scale, int window,
-                       int max_q, int heads, int block_size, hipStream_t stream) {
+                       int max_q, int heads, int block_size, int nsplit,
+                       float* part_acc, float* part_ml, hipStream_t stream) {
   constexpr int RANK = NT * 16, D = KS * 32;
   const size_t smem = sizeof(bf16) * (LM_KT * (D + LM_KPAD) + RANK * LM_VROW);
   static bool configured = false;
@@ -240,11 +332,16 @@ static void launch_one(bf16* out, long o_st, long o_sh, const bf16* q_lat,
   }
   const int hpb = heads < LM_ROWS ? heads : LM_ROWS;
   const int tq = LM_ROWS / hpb;
-  dim3 grid((max_q + tq - 1) / tq, nseq, (heads + hpb - 1) / hpb);
+  dim3 grid(nsplit > 1 ? nsplit : (max_q + tq - 1) / tq, nseq, (heads + hpb - 1) / hpb);
   latent_attn_mfma_kernel<NT, KS><<<grid, LM_THREADS, smem, stream>>>(
       out, o_st, o_sh, q_lat, ql_st, ql_sh, q_rot, qr_st, qr_sh, cache,
       block_tables, bt_stride, qsl, seq_lens, sinks, scale, window, heads, tq,
-      hpb, block_size);
+      hpb, block_size, nsplit, part_acc, part_ml);
+  if (nsplit > 1) {
+    dim3 mg(nseq, heads);
+    latent_attn_merge_kernel<<<mg, 128, 0, stream>>>(out, o_st, o_sh, part_acc, part_ml,
+                                                    sinks, nsplit, heads, RANK);
+  }
 }
 
 void launch_latent_attn_mfma(bf16* out, long o_st, long o_sh, const bf16* q_lat,
@@ -254,14 +351,15 @@ void launch_latent_attn_mfma(bf16* out, long o_st, long o_sh, const bf16* q_lat,
                              const int* qsl, const int* seq_lens, int nseq,
                              const float* sinks, float scale, int window,
                              int max_q, int heads, int rank, int rot,
-                             int block_size, hipStream_t stream) {
+                             int block_size, int nsplit, float* part_acc,
+                             float* part_ml, hipStream_t stream) {
   const int nt = rank / 16, ks = (rank + rot) / 32;
 #define X(A, B)                                                               \
   if (nt == A && ks == B) {                                                   \
     launch_one<A, B>(out, o_st, o_sh, q_lat, ql_st, ql_sh, q_rot, qr_st,     \
                      qr_sh, cache, block_tables, bt_stride, qsl, seq_lens,    \
                      nseq, sinks, scale, window, max_q, heads, block_size,    \
-                     stream);                                                 \
+                     nsplit, part_acc, part_ml, stream);                      \
     return;                                                                   \
   }
   LM_SHAPES(X)

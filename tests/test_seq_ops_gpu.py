@@ -202,3 +202,27 @@ def test_latent_attention_mfma(rank, rot, heads, window, bs):
         q_lat[rows].float(), q_rot[rows].float(), cache.float(), tables,
         torch.arange(len(seqs) + 1, dtype=torch.int32), lens, scale, window, sinks)
     torch.testing.assert_close(out_d.cpu().float(), want_d, atol=3e-2, rtol=3e-2)
+
+
+@pytest.mark.parametrize("window", [0, 100, 700])
+def test_latent_decode_key_slices_and_padding_rows(window):
+    """Single-query steps slice long key ranges over workgroups and merge;
+    rows of length zero (padding of a captured bucket) come out as zeros."""
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(window)
+    rank, rot, heads, bs = 128, 64, 8, 16
+    lens = torch.tensor([900, 0, 1, 33, 0, 640], dtype=torch.int32)
+    nb = 64
+    cache = torch.randn(nb * len(lens), bs, rank + rot, generator=g).to(dtype)
+    tables = torch.arange(nb * len(lens), dtype=torch.int32).view(len(lens), nb)
+    q_lat = torch.randn(len(lens), heads, rank, generator=g).to(dtype)
+    q_rot = torch.randn(len(lens), heads, rot, generator=g).to(dtype)
+    sinks = torch.randn(heads, generator=g)
+    out = torch.full((len(lens), heads, rank), float("nan"), dtype=dtype, device="cuda")
+    ops.latent_attention_decode(q_lat.cuda(), q_rot.cuda(), cache.cuda(), tables.cuda(),
+                                lens.cuda(), 0.1, window, sinks.cuda(), out=out)
+    want = ref.latent_attention(
+        q_lat.float(), q_rot.float(), cache.float(), tables,
+        torch.arange(len(lens) + 1, dtype=torch.int32), lens, 0.1, window, sinks)
+    torch.testing.assert_close(out.cpu().float(), want, atol=3e-2, rtol=3e-2)
+    assert float(out[1].abs().max()) == 0.0 and float(out[4].abs().max()) == 0.0
