@@ -19,7 +19,8 @@ template <typename T>
 void launch_stream_add(float*, const T*, const T*, float, T*, long, hipStream_t);
 template <typename T>
 void launch_stream_add_rms_norm(float*, const T*, const float*, float, float,
-                                int, int, hipStream_t);
+                                int, int, T*, const float*, float, float,
+                                hipStream_t);
 template <typename T>
 void launch_softcap(float*, const T*, float, long, hipStream_t);
 template <typename T>
@@ -156,17 +157,31 @@ void stream_add(torch::Tensor x, torch::Tensor a, c10::optional<torch::Tensor> b
 }
 
 void stream_add_rms_norm(torch::Tensor x, torch::Tensor y, torch::Tensor weight,
-                         double eps, double mult) {
+                         double eps, double mult,
+                         c10::optional<torch::Tensor> next_out,
+                         c10::optional<torch::Tensor> next_weight,
+                         double next_eps, double next_offset) {
   check_f32(x, "x");
   check_f32(weight, "weight");
   const int width = x.size(-1);
   TORCH_CHECK(y.is_cuda() && y.is_contiguous() && y.numel() == x.numel() &&
               weight.numel() == width);
   const int rows = x.numel() / width;
+  TORCH_CHECK(next_out.has_value() == next_weight.has_value());
+  if (next_out.has_value()) {
+    check_f32(next_weight.value(), "next_weight");
+    TORCH_CHECK(next_weight.value().numel() == width &&
+                next_out.value().is_contiguous() &&
+                next_out.value().numel() == x.numel() &&
+                next_out.value().scalar_type() == y.scalar_type());
+  }
   DISPATCH_F32_BF16(y.scalar_type(), {
-    launch_stream_add_rms_norm<scalar_t>(ptr<float>(x), ptr<scalar_t>(y),
-                                         ptr<float>(weight), (float)eps,
-                                         (float)mult, rows, width, stream());
+    launch_stream_add_rms_norm<scalar_t>(
+        ptr<float>(x), ptr<scalar_t>(y), ptr<float>(weight), (float)eps,
+        (float)mult, rows, width,
+        next_out.has_value() ? ptr<scalar_t>(next_out.value()) : nullptr,
+        next_out.has_value() ? ptr<float>(next_weight.value()) : nullptr,
+        (float)next_eps, (float)next_offset, stream());
   });
 }
 

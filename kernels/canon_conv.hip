@@ -12,10 +12,35 @@
 // is shorter than taps-1, from old state row j + n — each thread walks j
 // upwards, so it reads row j + n before that row is overwritten.
 //
-// One thread per (row, channel): consecutive threads take consecutive channels,
+// One thread per (row, 4 channels) — or one channel when the width is not a
+// multiple of 4: consecutive threads take consecutive channels,
 // every load and store is coalesced; accumulation is f32.
 
 #include "common.h"
+
+template <typename T, int CH>
+DEVINLINE void load_ch(const T* p, float* v) {
+  if (CH == 4) {
+    if (sizeof(T) == 4) {
+      const float4 t = *reinterpret_cast<const float4*>(p);
+      v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+    } else {
+      const uint2 t = *reinterpret_cast<const uint2*>(p);
+      v[0] = __uint_as_float(t.x << 16);
+      v[1] = __uint_as_float(t.x & 0xffff0000u);
+      v[2] = __uint_as_float(t.y << 16);
+      v[3] = __uint_as_float(t.y & 0xffff0000u);
+    }
+  } else {
+    v[0] = ScalarOps<T>::to_f32(p[0]);
+  }
+}
+
+template <typename T, int CH>
+DEVINLINE void store_ch(T* p, const float* v) {
+#pragma unroll
+  for (int k = 0; k < CH; ++k) p[k] = ScalarOps<T>::from_f32(v[k]);
+}
 
 DEVINLINE int find_seq(const int* __restrict__ loc, int nseq, int row) {
   int lo = 0, hi = nseq;  // largest s with loc[s] <= row
@@ -26,7 +51,8 @@ DEVINLINE int find_seq(const int* __restrict__ loc, int nseq, int row) {
   return lo;
 }
 
-template <typename T>
+// CH channels per thread: 4 (8/16-byte accesses) when width % 4 == 0, else 1.
+template <typename T, int CH>
 __global__ void causal_conv_kernel(T* __restrict__ out, const T* __restrict__ h,
                                    const float* __restrict__ w,   // [W, taps]
                                    const T* __restrict__ state,   // [slots, taps-1, W]
@@ -35,31 +61,40 @@ __global__ void causal_conv_kernel(T* __restrict__ out, const T* __restrict__ h,
                                    const int* __restrict__ slots, int nseq,
                                    int width, int taps, int add_input) {
   const int row = blockIdx.x;
-  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  const int c = (blockIdx.y * blockDim.x + threadIdx.x) * CH;
   if (c >= width) return;
   const int s = find_seq(loc, nseq, row);
   const int slot = slots[s];
   const long o = (long)row * width + c;
+  float acc[CH];
   if (slot < 0) {  // padding row of a captured bucket
-    out[o] = ScalarOps<T>::from_f32(0.f);
+#pragma unroll
+    for (int k = 0; k < CH; ++k) acc[k] = 0.f;
+    store_ch<T, CH>(out + o, acc);
     return;
   }
   const int n = loc[s + 1] - loc[s];
   const int start = seq_lens[s] - n;
   const int p = start + (row - loc[s]);
   const T* st = state + (long)slot * (taps - 1) * width;
-  float acc = add_input ? ScalarOps<T>::to_f32(h[o]) : 0.f;
+  if (add_input) {
+    load_ch<T, CH>(h + o, acc);
+  } else {
+#pragma unroll
+    for (int k = 0; k < CH; ++k) acc[k] = 0.f;
+  }
   for (int j = 0; j < taps; ++j) {
     const int pj = p - (taps - 1) + j;
     if (pj < 0) continue;
-    float v;
+    float v[CH];
     if (pj >= start)
-      v = ScalarOps<T>::to_f32(h[(long)(loc[s] + pj - start) * width + c]);
+      load_ch<T, CH>(h + (long)(loc[s] + pj - start) * width + c, v);
     else
-      v = ScalarOps<T>::to_f32(st[(long)(pj - (start - (taps - 1))) * width + c]);
-    acc += w[c * taps + j] * v;
+      load_ch<T, CH>(st + (long)(pj - (start - (taps - 1))) * width + c, v);
+#pragma unroll
+    for (int k = 0; k < CH; ++k) acc[k] += w[(c + k) * taps + j] * v[k];
   }
-  out[o] = ScalarOps<T>::from_f32(acc);
+  store_ch<T, CH>(out + o, acc);
 }
 
 template <typename T>
@@ -96,9 +131,18 @@ void launch_causal_conv_state(T* out, const T* h, const float* w, T* state,
                               const int* slots, int rows, int nseq, int width,
                               int taps, int add_input, hipStream_t stream) {
   const int block = 256;
-  dim3 g1(rows, (width + block - 1) / block);
-  causal_conv_kernel<T><<<g1, block, 0, stream>>>(
-      out, h, w, state, loc, seq_lens, slots, nseq, width, taps, add_input);
+  const bool vec = width % 4 == 0 &&
+                   reinterpret_cast<uintptr_t>(h) % (4 * sizeof(T)) == 0 &&
+                   reinterpret_cast<uintptr_t>(state) % (4 * sizeof(T)) == 0;
+  if (vec) {
+    dim3 g1(rows, (width / 4 + block - 1) / block);
+    causal_conv_kernel<T, 4><<<g1, block, 0, stream>>>(
+        out, h, w, state, loc, seq_lens, slots, nseq, width, taps, add_input);
+  } else {
+    dim3 g1(rows, (width + block - 1) / block);
+    causal_conv_kernel<T, 1><<<g1, block, 0, stream>>>(
+        out, h, w, state, loc, seq_lens, slots, nseq, width, taps, add_input);
+  }
   if (taps > 1) {
     dim3 g2(nseq, (width + block - 1) / block);
     conv_state_update_kernel<T><<<g2, block, 0, stream>>>(

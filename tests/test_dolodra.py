@@ -144,7 +144,7 @@ def test_layer_by_layer(model, device):
     e = _engine(path, device)
     caps = []
     for layer in e.worker.model.layers:
-        layer.register_forward_hook(lambda m, i, o: caps.append(o.detach().double().cpu().clone()))
+        layer.register_forward_hook(lambda m, i, o: caps.append(o[0].detach().double().cpu().clone()))
     _feed(e, "a", toks, [13])
     want = []
     oracle.forward(cfg, w, toks, want)

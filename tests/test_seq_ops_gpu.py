@@ -25,9 +25,9 @@ def _need_ext():
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_elementwise_and_norms(dtype):
+@pytest.mark.parametrize("t,w", [(37, 200), (5, 199)])   # rows of 4-groups / odd rows
+def test_elementwise_and_norms(dtype, t, w):
     g = torch.Generator().manual_seed(0)
-    t, w = 37, 200
     x = torch.randn(t, w, generator=g) * 3
     a = torch.randn(t, w, generator=g).to(dtype)
     b = torch.randn(t, w, generator=g).to(dtype)
@@ -56,6 +56,12 @@ def test_elementwise_and_norms(dtype):
     ref.stream_add_rms_norm(x1, a, wt, 1e-6, 0.7)
     ops.stream_add_rms_norm(x2, ad, wd, 1e-6, 0.7)
     torch.testing.assert_close(x2.cpu(), x1, atol=2e-5, rtol=1e-5)
+    # the same with the following norm fused in
+    ref.stream_add_rms_norm(x1, b, wt, 1e-6, 0.3)
+    h2 = ops.stream_add_rms_norm(x2, bd, wd, 1e-6, 0.3, (wd, 1e-5, 1.0, dtype))
+    torch.testing.assert_close(x2.cpu(), x1, atol=2e-5, rtol=1e-5)
+    torch.testing.assert_close(h2.cpu().float(),
+                               ref.rms_norm_stream(x1, wt, 1e-5, 1.0, dtype).float(), **_tol(dtype))
 
     torch.testing.assert_close(
         ops.softcap(ad * 10, 15.0).cpu(), ref.softcap(a * 10, 15.0), atol=1e-5, rtol=1e-5)

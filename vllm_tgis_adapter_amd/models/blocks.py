@@ -191,7 +191,13 @@ class TokenSideInput(nn.Module):
             torch.empty(width, side_dim, dtype=dtype).normal_(0.0, 0.02), requires_grad=False)
         self.norm = _f32_param(width, fill=1.0)
 
-    def forward(self, x: torch.Tensor, x_cast: torch.Tensor, e: torch.Tensor) -> None:
+    def forward(self, x: torch.Tensor, x_cast: torch.Tensor, e: torch.Tensor,
+                next_norm: "StreamRMSNorm | None" = None):
+        """Updates x in place; with ``next_norm`` the norm that reads the
+        updated stream next is computed in the same kernel and returned."""
         g = ops.gelu_tanh(ops.linear(x_cast, self.gate), mul=e)
         y = ops.linear(g, self.proj)
-        ops.stream_add_rms_norm(x, y, self.norm, self.eps, self.mult)
+        nn_ = None
+        if next_norm is not None:
+            nn_ = (next_norm.weight, next_norm.eps, next_norm.weight_offset, next_norm.dtype)
+        return ops.stream_add_rms_norm(x, y, self.norm, self.eps, self.mult, nn_)

@@ -141,17 +141,22 @@ class DolodraLayer(nn.Module):
         self.mlp = DenseMLP(width, spec.ff, dtype) if spec.ff else None
         self.side = TokenSideInput(width, side_dim, eps, mult, dtype) if side_dim else None
 
-    def forward(self, x, positions, cache, meta, side_e):
+    def forward(self, x, positions, cache, meta, side_e, h=None, next_norm=None):
+        """x: f32 stream (updated in place).  h: this layer's norm1 output when
+        the previous layer already produced it.  Returns (x, h_next): h_next is
+        next_norm(x) computed inside the side-input kernel, or None."""
         latent, conv_state = cache
-        h = self.norm1(x)
+        if h is None:
+            h = self.norm1(x)
         hm = self.canon(h, conv_state, meta) if self.canon is not None else h
         mix = self.mix(hm, positions, latent, meta)
         ff = self.mlp(h) if self.mlp is not None else None
         xc = ops.stream_add(x, mix, ff, self.mult,
                             cast_dtype=self.dtype if self.side is not None else None)
+        h_next = None
         if self.side is not None:
-            self.side(x, xc, side_e)
-        return x
+            h_next = self.side(x, xc, side_e, next_norm)
+        return x, h_next
 
 
 class DolodraForCausalLM(nn.Module):
@@ -228,10 +233,13 @@ class DolodraForCausalLM(nn.Module):
         x = ops.embedding_scaled(input_ids, self.embed, self.embed_scale)   # f32 [T, W]
         side = F.embedding(input_ids, self.side_embed) if self.side_dim else None
         sd = self.side_dim
+        h = None
+        last = len(self.layers) - 1
         for i, layer in enumerate(self.layers):
             e = side[:, i * sd:(i + 1) * sd] if sd else None
-            x = layer(x, positions, kv_caches[i], meta, e)
-        return self.final_norm(x)
+            nxt = self.layers[i + 1].norm1 if i < last else self.final_norm
+            x, h = layer(x, positions, kv_caches[i], meta, e, h, nxt)
+        return h if h is not None else self.final_norm(x)
 
     def compute_logits(self, hidden: torch.Tensor) -> torch.Tensor:
         logits = self.lm_head(hidden)

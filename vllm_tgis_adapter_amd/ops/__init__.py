@@ -491,12 +491,26 @@ def stream_add(x: torch.Tensor, a: torch.Tensor, b: torch.Tensor | None,
 
 
 def stream_add_rms_norm(x: torch.Tensor, y: torch.Tensor, weight: torch.Tensor,
-                        eps: float, mult: float) -> None:
-    """x (f32, in place) += mult * y / rms(y) * weight."""
+                        eps: float, mult: float, next_norm=None):
+    """x (f32, in place) += mult * y / rms(y) * weight.
+
+    ``next_norm`` = (weight, eps, weight_offset, dtype) fuses the following
+    norm of the updated stream into the same pass and returns its output."""
     if x.numel() and _native_seq(x):
-        _S.stream_add_rms_norm(x, y, weight, float(eps), float(mult))
-        return
+        if next_norm is None:
+            _S.stream_add_rms_norm(x, y, weight, float(eps), float(mult),
+                                   None, None, 0.0, 0.0)
+            return None
+        nw, neps, noff, ndtype = next_norm
+        out = torch.empty(x.shape, dtype=ndtype, device=x.device)
+        _S.stream_add_rms_norm(x, y, weight, float(eps), float(mult), out, nw,
+                               float(neps), float(noff))
+        return out
     reference.stream_add_rms_norm(x, y, weight, eps, mult)
+    if next_norm is None:
+        return None
+    nw, neps, noff, ndtype = next_norm
+    return reference.rms_norm_stream(x, nw, neps, noff, ndtype)
 
 
 def softcap(logits: torch.Tensor, cap: float) -> torch.Tensor:
