@@ -35,12 +35,17 @@ typedef __hip_bfloat16 bf16;
 #define LM_KT 32
 #define LM_KPAD 8
 #define LM_VROW 40
+#define LM_BT_MAX 512    // block-table entries kept in LDS per workgroup
 
 DEVINLINE short f32_to_bf16_bits(float x) {
   return __builtin_bit_cast(short, __float2bfloat16(x));
 }
 
-template <int NT, int KS>
+// DS = 1: the four waves own four 16-row tiles (64 rows).  DS = 4: at most 16
+// rows (a single query of <= 16 heads): every wave scores the same row tile and
+// owns a quarter of the latent dims for the value product — a quarter of the
+// accumulators per wave, so two workgroups fit a CU.
+template <int NT, int KS, int DS>
 __global__ __launch_bounds__(LM_THREADS) void latent_attn_mfma_kernel(
     bf16* __restrict__ out, long o_st, long o_sh,
     const bf16* __restrict__ q_lat, long ql_st, long ql_sh,
@@ -53,9 +58,11 @@ __global__ __launch_bounds__(LM_THREADS) void latent_attn_mfma_kernel(
   constexpr int RANK = NT * 16;
   constexpr int D = KS * 32;
   constexpr int KROW = D + LM_KPAD;
+  constexpr int NTW = NT / DS;     // accumulator tiles per wave
   extern __shared__ char lds_raw[];
   bf16* k_img = reinterpret_cast<bf16*>(lds_raw);   // [32][KROW]
   bf16* v_img = k_img + LM_KT * KROW;               // [RANK][LM_VROW]
+  int* bt_s = reinterpret_cast<int*>(v_img + RANK * LM_VROW);   // [LM_BT_MAX]
 
   const int seq = blockIdx.y;
   int q0, nq;
@@ -78,7 +85,9 @@ __global__ __launch_bounds__(LM_THREADS) void latent_attn_mfma_kernel(
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n = lane & 15, g = lane >> 4;
-  const int r = wave * 16 + n;
+  const int rt = (DS == 1) ? wave : 0;   // row tile of this wave
+  const int dp = (DS == 1) ? 0 : wave;   // dim part of this wave
+  const int r = rt * 16 + n;
   const bool row_ok = r < nrows;
   const int tl = row_ok ? r / nh : 0;
   const int head = h0 + (row_ok ? r % nh : 0);
@@ -86,9 +95,9 @@ __global__ __launch_bounds__(LM_THREADS) void latent_attn_mfma_kernel(
   bf16* orow = out + qrow * o_st + head * o_sh;
 
   if (slen <= 0) {   // padding row of a captured bucket
-    if (row_ok && split == 0)
+    if (row_ok && split == 0 && dp == 0)
       for (int k = g; k < RANK; k += 4) orow[k] = __float2bfloat16(0.f);
-    if (nsplit > 1 && row_ok && g == 0) {
+    if (nsplit > 1 && row_ok && g == 0 && dp == 0) {
       float* ml = part_ml + (((long)seq * nsplit + split) * heads + head) * 2;
       ml[0] = -INFINITY;
       ml[1] = -1.f;     // tells the merge: nothing to do, the row is zero already
@@ -107,7 +116,24 @@ __global__ __launch_bounds__(LM_THREADS) void latent_attn_mfma_kernel(
   const int qpos = pos0 + tl;
   const int klo = (window > 0) ? qpos - window + 1 : 0;
   const int* bt = block_tables + (long)seq * bt_stride;
-  const bool wave_active = wave * 16 < nrows;
+  const bool wave_active = rt * 16 < nrows;
+
+  // The block-table entries of this workgroup's key range go to LDS once: a
+  // tile's row addresses then depend on no global load (a table read in the
+  // loop would put two memory latencies in series per tile).
+  const int bs_shift = ((block_size & (block_size - 1)) == 0) ? __ffs(block_size) - 1 : -1;
+  const int blk0 = (kstart < kend ? kstart : 0) / block_size;
+  const int nblk = (kstart < kend) ? (kend - 1) / block_size - blk0 + 1 : 0;
+  const bool bt_in_lds = nblk <= LM_BT_MAX;
+  if (bt_in_lds)
+    for (int i = tid; i < nblk; i += LM_THREADS) bt_s[i] = bt[blk0 + i];
+  __syncthreads();
+  auto row_offset = [&](int kk) -> long {
+    const int b = (bs_shift >= 0) ? (kk >> bs_shift) : (kk / block_size);
+    const int in = kk - b * block_size;
+    const int phys = bt_in_lds ? bt_s[b - blk0] : bt[b];
+    return ((long)phys * block_size + in) * D;
+  };
 
   bf16x8_t qf[KS];
 #pragma unroll
@@ -123,9 +149,9 @@ __global__ __launch_bounds__(LM_THREADS) void latent_attn_mfma_kernel(
     qf[ks] = v;
   }
 
-  f32x4_t acc[NT];
+  f32x4_t acc[NTW];
 #pragma unroll
-  for (int i = 0; i < NT; ++i) acc[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  for (int i = 0; i < NTW; ++i) acc[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   float m_run = -INFINITY, l_part = 0.f;
 
   // global loads of a tile are issued one tile ahead and parked in registers:
@@ -140,8 +166,7 @@ __global__ __launch_bounds__(LM_THREADS) void latent_attn_mfma_kernel(
       if (c < LM_KT * CPR) {
         const int key = c / CPR, ch = c - key * CPR;
         const int kk = min(base + key, kend - 1);
-        const long off = ((long)bt[kk / block_size] * block_size + (kk % block_size)) * D + ch * 8;
-        pre[i] = *reinterpret_cast<const bf16x8_t*>(cache + off);
+        pre[i] = *reinterpret_cast<const bf16x8_t*>(cache + row_offset(kk) + ch * 8);
       }
     }
   };
@@ -207,15 +232,15 @@ __global__ __launch_bounds__(LM_THREADS) void latent_attn_mfma_kernel(
     l_part = l_part * alpha + ps;
     m_run = m_new;
 #pragma unroll
-    for (int i = 0; i < NT; ++i) {
+    for (int i = 0; i < NTW; ++i) {
       acc[i][0] *= alpha; acc[i][1] *= alpha; acc[i][2] *= alpha; acc[i][3] *= alpha;
     }
     __syncthreads();   // V^T image complete
     if (wave_active) {
 #pragma unroll
-      for (int dt = 0; dt < NT; ++dt) {
+      for (int dt = 0; dt < NTW; ++dt) {
         const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(
-            v_img + (dt * 16 + n) * LM_VROW + g * 8);
+            v_img + ((dp * NTW + dt) * 16 + n) * LM_VROW + g * 8);
         acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb, acc[dt], 0, 0, 0);
       }
     }
@@ -228,13 +253,13 @@ __global__ __launch_bounds__(LM_THREADS) void latent_attn_mfma_kernel(
     // unnormalised slice result; the merge kernel adds the sink and divides
     if (row_ok) {
       const long pr = ((long)seq * nsplit + split) * heads + head;
-      if (g == 0) {
+      if (g == 0 && dp == 0) {
         part_ml[pr * 2] = m_run;
         part_ml[pr * 2 + 1] = l;
       }
 #pragma unroll
-      for (int dt = 0; dt < NT; ++dt)
-        *reinterpret_cast<f32x4_t*>(part_acc + pr * RANK + dt * 16 + 4 * g) = acc[dt];
+      for (int dt = 0; dt < NTW; ++dt)
+        *reinterpret_cast<f32x4_t*>(part_acc + pr * RANK + (dp * NTW + dt) * 16 + 4 * g) = acc[dt];
     }
     return;
   }
@@ -248,11 +273,11 @@ __global__ __launch_bounds__(LM_THREADS) void latent_attn_mfma_kernel(
   const float inv = (l > 0.f) ? rescale / l : 0.f;
   if (row_ok) {
 #pragma unroll
-    for (int dt = 0; dt < NT; ++dt) {
+    for (int dt = 0; dt < NTW; ++dt) {
       union { short s[4]; uint2 v; } o;
 #pragma unroll
       for (int i = 0; i < 4; ++i) o.s[i] = f32_to_bf16_bits(acc[dt][i] * inv);
-      *reinterpret_cast<uint2*>(orow + dt * 16 + 4 * g) = o.v;
+      *reinterpret_cast<uint2*>(orow + (dp * NTW + dt) * 16 + 4 * g) = o.v;
     }
   }
 }
@@ -294,7 +319,9 @@ __global__ void latent_attn_merge_kernel(bf16* __restrict__ out, long o_st, long
 int latent_decode_num_splits(int nseq, int heads, int max_keys) {
   const int groups = (heads + LM_ROWS - 1) / LM_ROWS;
   const int tiles = (max_keys + LM_KT - 1) / LM_KT;
-  int want = (256 + nseq * groups - 1) / (nseq * groups);
+  // the dim-split variant (<= 16 heads) fits two workgroups per CU
+  const int target = heads <= 16 ? 512 : 256;
+  int want = (target + nseq * groups - 1) / (nseq * groups);
   if (want > tiles / 2) want = tiles / 2;   // at least two tiles per slice
   if (want > 32) want = 32;
   return want < 1 ? 1 : want;
@@ -314,7 +341,7 @@ bool latent_prefill_mfma_usable(int rank, int rot, int block_size) {
   return false;
 }
 
-template <int NT, int KS>
+template <int NT, int KS, int DS>
 static void launch_one(bf16* out, long o_st, long o_sh, const bf16* q_lat,
                        long ql_st, long ql_sh, const bf16* q_rot, long qr_st,
                        long qr_sh, const bf16* cache, const int* block_tables,
@@ -323,17 +350,18 @@ static void launch_one(bf16* out, long o_st, long o_sh, const bf16* q_lat,
                        int max_q, int heads, int block_size, int nsplit,
                        float* part_acc, float* part_ml, hipStream_t stream) {
   constexpr int RANK = NT * 16, D = KS * 32;
-  const size_t smem = sizeof(bf16) * (LM_KT * (D + LM_KPAD) + RANK * LM_VROW);
+  const size_t smem = sizeof(bf16) * (LM_KT * (D + LM_KPAD) + RANK * LM_VROW) +
+                      sizeof(int) * LM_BT_MAX;
   static bool configured = false;
   if (!configured) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&latent_attn_mfma_kernel<NT, KS>),
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&latent_attn_mfma_kernel<NT, KS, DS>),
                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     configured = true;
   }
   const int hpb = heads < LM_ROWS ? heads : LM_ROWS;
   const int tq = LM_ROWS / hpb;
   dim3 grid(nsplit > 1 ? nsplit : (max_q + tq - 1) / tq, nseq, (heads + hpb - 1) / hpb);
-  latent_attn_mfma_kernel<NT, KS><<<grid, LM_THREADS, smem, stream>>>(
+  latent_attn_mfma_kernel<NT, KS, DS><<<grid, LM_THREADS, smem, stream>>>(
       out, o_st, o_sh, q_lat, ql_st, ql_sh, q_rot, qr_st, qr_sh, cache,
       block_tables, bt_stride, qsl, seq_lens, sinks, scale, window, heads, tq,
       hpb, block_size, nsplit, part_acc, part_ml);
@@ -354,12 +382,20 @@ void launch_latent_attn_mfma(bf16* out, long o_st, long o_sh, const bf16* q_lat,
                              int block_size, int nsplit, float* part_acc,
                              float* part_ml, hipStream_t stream) {
   const int nt = rank / 16, ks = (rank + rot) / 32;
+  // one query per sequence and at most one 16-row tile of heads
+  const bool dim_split = (qsl == nullptr) && heads <= 16;
 #define X(A, B)                                                               \
   if (nt == A && ks == B) {                                                   \
-    launch_one<A, B>(out, o_st, o_sh, q_lat, ql_st, ql_sh, q_rot, qr_st,     \
-                     qr_sh, cache, block_tables, bt_stride, qsl, seq_lens,    \
-                     nseq, sinks, scale, window, max_q, heads, block_size,    \
-                     nsplit, part_acc, part_ml, stream);                      \
+    if (dim_split && A % 4 == 0)                                              \
+      launch_one<A, B, (A % 4 == 0 ? 4 : 1)>(                                 \
+          out, o_st, o_sh, q_lat, ql_st, ql_sh, q_rot, qr_st, qr_sh, cache,  \
+          block_tables, bt_stride, qsl, seq_lens, nseq, sinks, scale, window, \
+          max_q, heads, block_size, nsplit, part_acc, part_ml, stream);       \
+    else                                                                      \
+      launch_one<A, B, 1>(                                                    \
+          out, o_st, o_sh, q_lat, ql_st, ql_sh, q_rot, qr_st, qr_sh, cache,  \
+          block_tables, bt_stride, qsl, seq_lens, nseq, sinks, scale, window, \
+          max_q, heads, block_size, nsplit, part_acc, part_ml, stream);       \
     return;                                                                   \
   }
   LM_SHAPES(X)
