@@ -52,7 +52,10 @@ DEVINLINE int find_seq(const int* __restrict__ loc, int nseq, int row) {
 }
 
 // CH channels per thread: 4 (8/16-byte accesses) when width % 4 == 0, else 1.
-template <typename T, int CH>
+// TAPS > 0: tap count known at compile time — the thread's CH x TAPS weights
+// are one contiguous run fetched with 16-byte loads into registers; TAPS == 0
+// reads them one by one for any tap count.
+template <typename T, int CH, int TAPS>
 __global__ void causal_conv_kernel(T* __restrict__ out, const T* __restrict__ h,
                                    const float* __restrict__ w,   // [W, taps]
                                    const T* __restrict__ state,   // [slots, taps-1, W]
@@ -77,13 +80,22 @@ __global__ void causal_conv_kernel(T* __restrict__ out, const T* __restrict__ h,
   const int start = seq_lens[s] - n;
   const int p = start + (row - loc[s]);
   const T* st = state + (long)slot * (taps - 1) * width;
+  float wreg[CH * (TAPS > 0 ? TAPS : 1)];
+  if (TAPS > 0 && CH == 4) {
+#pragma unroll
+    for (int i = 0; i < TAPS; ++i) {
+      const float4 t = reinterpret_cast<const float4*>(w + (long)c * TAPS)[i];
+      wreg[4 * i] = t.x; wreg[4 * i + 1] = t.y; wreg[4 * i + 2] = t.z; wreg[4 * i + 3] = t.w;
+    }
+  }
   if (add_input) {
     load_ch<T, CH>(h + o, acc);
   } else {
 #pragma unroll
     for (int k = 0; k < CH; ++k) acc[k] = 0.f;
   }
-  for (int j = 0; j < taps; ++j) {
+#pragma unroll
+  for (int j = 0; j < (TAPS > 0 ? TAPS : taps); ++j) {
     const int pj = p - (taps - 1) + j;
     if (pj < 0) continue;
     float v[CH];
@@ -92,7 +104,10 @@ __global__ void causal_conv_kernel(T* __restrict__ out, const T* __restrict__ h,
     else
       load_ch<T, CH>(st + (long)(pj - (start - (taps - 1))) * width + c, v);
 #pragma unroll
-    for (int k = 0; k < CH; ++k) acc[k] += w[(c + k) * taps + j] * v[k];
+    for (int k = 0; k < CH; ++k) {
+      const float wk = (TAPS > 0 && CH == 4) ? wreg[k * TAPS + j] : w[(c + k) * taps + j];
+      acc[k] += wk * v[k];
+    }
   }
   store_ch<T, CH>(out + o, acc);
 }
@@ -133,14 +148,23 @@ void launch_causal_conv_state(T* out, const T* h, const float* w, T* state,
   const int block = 256;
   const bool vec = width % 4 == 0 &&
                    reinterpret_cast<uintptr_t>(h) % (4 * sizeof(T)) == 0 &&
-                   reinterpret_cast<uintptr_t>(state) % (4 * sizeof(T)) == 0;
+                   reinterpret_cast<uintptr_t>(state) % (4 * sizeof(T)) == 0 &&
+                   reinterpret_cast<uintptr_t>(w) % 16 == 0;
   if (vec) {
     dim3 g1(rows, (width / 4 + block - 1) / block);
-    causal_conv_kernel<T, 4><<<g1, block, 0, stream>>>(
-        out, h, w, state, loc, seq_lens, slots, nseq, width, taps, add_input);
+#define CONV_LAUNCH(TP)                                                        \
+    causal_conv_kernel<T, 4, TP><<<g1, block, 0, stream>>>(                    \
+        out, h, w, state, loc, seq_lens, slots, nseq, width, taps, add_input)
+    switch (taps) {
+      case 2: CONV_LAUNCH(2); break;
+      case 3: CONV_LAUNCH(3); break;
+      case 4: CONV_LAUNCH(4); break;
+      default: CONV_LAUNCH(0); break;
+    }
+#undef CONV_LAUNCH
   } else {
     dim3 g1(rows, (width + block - 1) / block);
-    causal_conv_kernel<T, 1><<<g1, block, 0, stream>>>(
+    causal_conv_kernel<T, 1, 0><<<g1, block, 0, stream>>>(
         out, h, w, state, loc, seq_lens, slots, nseq, width, taps, add_input);
   }
   if (taps > 1) {

@@ -41,10 +41,10 @@ DEVINLINE short f32_to_bf16_bits(float x) {
   return __builtin_bit_cast(short, __float2bfloat16(x));
 }
 
-// DS = 1: the four waves own four 16-row tiles (64 rows).  DS = 4: at most 16
-// rows (a single query of <= 16 heads): every wave scores the same row tile and
-// owns a quarter of the latent dims for the value product — a quarter of the
-// accumulators per wave, so two workgroups fit a CU.
+// DS = 1: the four waves own four 16-row tiles (64 rows).  DS = 4 / 2: at most
+// 16 / 32 rows (a single query of <= 16 / 32 heads): the waves that share a row
+// tile all score it and each owns a quarter / half of the latent dims for the
+// value product — fewer accumulators per wave, so two workgroups fit a CU.
 template <int NT, int KS, int DS>
 __global__ __launch_bounds__(LM_THREADS) void latent_attn_mfma_kernel(
     bf16* __restrict__ out, long o_st, long o_sh,
@@ -85,8 +85,9 @@ __global__ __launch_bounds__(LM_THREADS) void latent_attn_mfma_kernel(
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n = lane & 15, g = lane >> 4;
-  const int rt = (DS == 1) ? wave : 0;   // row tile of this wave
-  const int dp = (DS == 1) ? 0 : wave;   // dim part of this wave
+  constexpr int RT = 4 / DS;
+  const int rt = wave % RT;              // row tile of this wave
+  const int dp = wave / RT;              // dim part of this wave
   const int r = rt * 16 + n;
   const bool row_ok = r < nrows;
   const int tl = row_ok ? r / nh : 0;
@@ -319,8 +320,8 @@ __global__ void latent_attn_merge_kernel(bf16* __restrict__ out, long o_st, long
 int latent_decode_num_splits(int nseq, int heads, int max_keys) {
   const int groups = (heads + LM_ROWS - 1) / LM_ROWS;
   const int tiles = (max_keys + LM_KT - 1) / LM_KT;
-  // the dim-split variant (<= 16 heads) fits two workgroups per CU
-  const int target = heads <= 16 ? 512 : 256;
+  // the dim-split variants (<= 32 heads) fit two workgroups per CU
+  const int target = heads <= 32 ? 512 : 256;
   int want = (target + nseq * groups - 1) / (nseq * groups);
   if (want > tiles / 2) want = tiles / 2;   // at least two tiles per slice
   if (want > 32) want = 32;
@@ -383,11 +384,16 @@ void launch_latent_attn_mfma(bf16* out, long o_st, long o_sh, const bf16* q_lat,
                              float* part_ml, hipStream_t stream) {
   const int nt = rank / 16, ks = (rank + rot) / 32;
   // one query per sequence and at most one 16-row tile of heads
-  const bool dim_split = (qsl == nullptr) && heads <= 16;
+  const int dim_split = (qsl != nullptr || heads > 32) ? 1 : (heads <= 16 ? 4 : 2);
 #define X(A, B)                                                               \
   if (nt == A && ks == B) {                                                   \
-    if (dim_split && A % 4 == 0)                                              \
+    if (dim_split == 4 && A % 4 == 0)                                         \
       launch_one<A, B, (A % 4 == 0 ? 4 : 1)>(                                 \
+          out, o_st, o_sh, q_lat, ql_st, ql_sh, q_rot, qr_st, qr_sh, cache,  \
+          block_tables, bt_stride, qsl, seq_lens, nseq, sinks, scale, window, \
+          max_q, heads, block_size, nsplit, part_acc, part_ml, stream);       \
+    else if (dim_split >= 2)                                                  \
+      launch_one<A, B, 2>(                                                    \
           out, o_st, o_sh, q_lat, ql_st, ql_sh, q_rot, qr_st, qr_sh, cache,  \
           block_tables, bt_stride, qsl, seq_lens, nseq, sinks, scale, window, \
           max_q, heads, block_size, nsplit, part_acc, part_ml, stream);       \

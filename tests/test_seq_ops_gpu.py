@@ -71,7 +71,7 @@ def test_elementwise_and_norms(dtype, t, w):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("taps", [1, 2, 3, 5])
+@pytest.mark.parametrize("taps", [1, 2, 3, 4, 5])
 def test_causal_conv_state(dtype, taps):
     g = torch.Generator().manual_seed(taps)
     w = 72
