@@ -357,3 +357,67 @@ def test_greedy_generation_matches_oracle(model, device):
                 break
         assert done[rid] == seq[len(p):], rid
     assert e.state_manager.num_free_slots == 3
+
+
+# -- tensor parallel (gloo, two ranks on the CPU) ------------------------------
+
+
+def _tp_worker(rank, world, port, q):
+    import os
+
+    try:
+        os.environ.update(MASTER_ADDR="127.0.0.1", MASTER_PORT=str(port), RANK=str(rank),
+                          WORLD_SIZE=str(world))
+        from vllm_tgis_adapter_amd.parallel import init_distributed
+
+        init_distributed(world, rank=rank, device="cpu", backend="gloo")
+        from vllm_tgis_adapter_amd.engine.worker import Worker
+
+        mc = ModelConfig.from_model_arg(os.environ["DOLODRA_TP_MODEL"], dtype="float32")
+        cfg = EngineConfig(
+            model_config=mc,
+            cache_config=CacheConfig(block_size=4, num_gpu_blocks=48),
+            scheduler_config=SchedulerConfig(max_num_seqs=3, max_num_batched_tokens=1 << 20),
+            device="cpu", tensor_parallel_size=world, enforce_eager=True)
+        if rank == 0:
+            e = LLMEngine(cfg)
+            a, b = _tokens(21, mc.vocab_size, 41), _tokens(9, mc.vocab_size, 42)
+            got_a = [e.replay_step([("a", a[:8], list(range(8))), ("b", b[:2], [0, 1])])]
+            got_a.append(e.replay_step([("a", a[8:9], [0]), ("b", b[2:], list(range(7)))], ["b"]))
+            got_a.append(e.replay_step([("a", a[9:], list(range(12)))], ["a"]))
+            e.worker.stop_workers()
+            rows_a = torch.cat([got_a[0][:8], got_a[1][:1], got_a[2]]).double()
+            rows_b = torch.cat([got_a[0][8:], got_a[1][1:]]).double()
+            q.put((rank, (rows_a, rows_b)))
+        else:
+            w = Worker(cfg)
+            w.init_kv_cache()
+            w.worker_loop()
+            q.put((rank, None))
+    except Exception:
+        import traceback
+
+        q.put((rank, "ERROR " + traceback.format_exc()))
+    finally:
+        import torch.distributed as dist
+
+        if dist.is_initialized():
+            dist.destroy_process_group()
+
+
+def test_tensor_parallel_two_ranks(tmp_path, monkeypatch):
+    """Heads, feed-forward and vocabulary sharded over two ranks (latent rows
+    and conv state replicated) reproduce the oracle."""
+    from test_distributed import _run_spawn
+
+    cfg = oracle.make_config(layers=[
+        dict(heads=4, dim=8, rot_dim=4, vdim=6, kv_rank=20, window=5, ff=40),
+        dict(heads=2, dim=6, rot_dim=4, vdim=8, kv_rank=20, window=9, ff=0, kv_from=0),
+        dict(heads=2, dim=10, rot_dim=8, vdim=6, kv_rank=12, window=3, ff=24)], vocab=98)
+    w = oracle.make_weights(cfg, seed=2)
+    path = oracle.save_model(tmp_path / "tp", cfg, w)
+    monkeypatch.setenv("DOLODRA_TP_MODEL", path)
+    res = _run_spawn(_tp_worker, 2, timeout=300)
+    rows_a, rows_b = res[0]
+    _close(rows_a, oracle.forward(cfg, w, _tokens(21, 98, 41)))
+    _close(rows_b, oracle.forward(cfg, w, _tokens(9, 98, 42)))
