@@ -259,6 +259,48 @@ def test_bf16_stays_near_oracle(model, device):
     _close(b, want, "bfloat16")
 
 
+@pytest.mark.gpu
+def test_captured_decode_steps_match_eager(model):
+    """Decode-only steps replay captured graphs; replays interleaved with eager
+    prompt portions and with slot / block reuse equal the eager engine."""
+    cfg, w, path = model
+    toks = {k: _tokens(n, cfg["vocab"], 50 + i) for i, (k, n) in
+            enumerate([("a", 25), ("b", 17), ("c", 22)])}
+    outs = []
+    for eager in (True, False):
+        e = _engine(path, "cuda", blocks=24, slots=2, eager=eager)
+        if not eager:
+            assert e.worker.graph_runner is not None and e.worker.graph_runner.graphs
+        got = {k: [] for k in toks}
+        at = {k: 0 for k in toks}
+
+        def step(parts, done=()):
+            entries = [(k, toks[k][at[k]:at[k] + n], list(range(n))) for k, n in parts]
+            lg = e.replay_step(entries, list(done)).double().cpu()
+            o = 0
+            for k, n in parts:
+                got[k].append(lg[o:o + n])
+                at[k] += n
+                o += n
+
+        step([("a", 9), ("b", 5)])
+        for _ in range(6):
+            step([("a", 1), ("b", 1)])             # graph bucket 2
+        step([("a", 1), ("b", 6)], done=["b"])     # eager, mixed
+        for _ in range(4):
+            step([("a", 1)])                       # graph bucket 1
+        step([("c", 20), ("a", 1)])                # c takes b's slot and blocks
+        for _ in range(2):
+            step([("a", 1), ("c", 1)])
+        step([("a", 2)], done=["a"])
+        outs.append({k: torch.cat(v) for k, v in got.items()})
+    for k in ("a", "b"):
+        want = oracle.forward(cfg, w, toks[k])
+        _close(outs[1][k], want)
+        _close(outs[0][k], outs[1][k])
+    _close(outs[1]["c"], oracle.forward(cfg, w, toks["c"])[:22])
+
+
 # -- a key that must / must not be seen ---------------------------------------
 
 
