@@ -463,3 +463,49 @@ def test_tensor_parallel_two_ranks(tmp_path, monkeypatch):
     rows_a, rows_b = res[0]
     _close(rows_a, oracle.forward(cfg, w, _tokens(21, 98, 41)))
     _close(rows_b, oracle.forward(cfg, w, _tokens(9, 98, 42)))
+
+
+# -- the serving entry: command-line flags -> async engine ---------------------
+
+
+def test_served_from_command_line_flags(tmp_path):
+    """A Dolodra directory given as --model goes through the server's flag
+    parsing into the async engine and streams greedy tokens equal to the
+    oracle's, concurrent requests included."""
+    import asyncio
+
+    from vllm_tgis_adapter_amd.__main__ import parse_args
+    from vllm_tgis_adapter_amd.engine.async_engine import AsyncLLMEngine
+    from vllm_tgis_adapter_amd.tgis_utils.args import engine_config_from_args
+
+    cfg = oracle.make_config(vocab=300)    # room for the byte-level test tokenizer
+    w = oracle.make_weights(cfg, seed=5)
+    path = oracle.save_model(tmp_path / "served", cfg, w)
+    args = parse_args(["--model", path, "--dtype", "float32", "--max-num-seqs", "2",
+                       "--num-gpu-blocks", "64", "--block-size", "8", "--device", "cpu"])
+    engine = AsyncLLMEngine(engine_config_from_args(args))
+    prompts = {"x": _tokens(12, 300, 61), "y": _tokens(5, 300, 62), "z": _tokens(9, 300, 63)}
+
+    async def one(rid):
+        last = None
+        async for out in engine.generate(
+                {"prompt_token_ids": prompts[rid]},
+                SamplingParams(temperature=0.0, max_tokens=5), request_id=rid):
+            last = out
+        return rid, list(last.outputs[0].token_ids)
+
+    async def main():
+        return dict(await asyncio.gather(*[one(r) for r in prompts]))
+
+    try:
+        got = asyncio.run(main())
+    finally:
+        engine.shutdown()
+    eos = engine.engine.eos_token_id
+    for rid, p in prompts.items():
+        seq = list(p)
+        for _ in range(5):
+            seq.append(int(oracle.forward(cfg, w, seq)[-1].argmax()))
+            if seq[-1] == eos:
+                break
+        assert got[rid] == seq[len(p):], rid
