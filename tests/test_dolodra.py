@@ -509,3 +509,33 @@ def test_served_from_command_line_flags(tmp_path):
             if seq[-1] == eos:
                 break
         assert got[rid] == seq[len(p):], rid
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_matrix_core_shapes(tmp_path, device, dtype):
+    """Latent sizes on the bf16 matrix-core kernel's list (64+32, 32+32 with more
+    than 16 heads, 128+64) through the engine: whole, portions, decode, batch."""
+    cfg = oracle.make_config(
+        width=64, vocab=211, taps=4, side_dim=8,
+        layers=[dict(heads=4, dim=16, rot_dim=32, vdim=16, kv_rank=64, window=11, ff=96),
+                dict(heads=20, dim=8, rot_dim=32, vdim=8, kv_rank=64, window=37, ff=0, kv_from=0),
+                dict(heads=20, dim=8, rot_dim=32, vdim=8, kv_rank=32, window=6, ff=64),
+                dict(heads=2, dim=32, rot_dim=64, vdim=32, kv_rank=128, window=70, ff=0)])
+    w = oracle.make_weights(cfg, seed=21)
+    path = oracle.save_model(tmp_path / "mc", cfg, w)
+    a, b = _tokens(45, 211, 71), _tokens(19, 211, 72)
+    want_a, want_b = oracle.forward(cfg, w, a), oracle.forward(cfg, w, b)
+    e = _engine(path, device, dtype=dtype, block_size=16, blocks=12, slots=2, eager=False)
+    _close(_feed(e, "w", a, [45]), want_a, dtype)
+    got_a, got_b = [], []
+    lg = e.replay_step([("a", a[:30], list(range(30))), ("b", b[:2], [0, 1])])
+    got_a.append(lg[:30]); got_b.append(lg[30:])
+    for i in range(15):
+        lg = e.replay_step([("b", b[2 + i:3 + i], [0]), ("a", a[30 + i:31 + i], [0])],
+                           ["a"] if i == 14 else [])
+        got_b.append(lg[:1]); got_a.append(lg[1:])
+    lg = e.replay_step([("b", b[17:], [0, 1])], ["b"])
+    got_b.append(lg)
+    _close(torch.cat(got_a).double().cpu(), want_a, dtype)
+    _close(torch.cat(got_b).double().cpu(), want_b, dtype)
