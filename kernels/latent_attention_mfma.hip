@@ -19,6 +19,10 @@
 //           same slot order so its A fragments are single 16-byte reads)
 //   values  O^T += V^T . P^T, rank/16 accumulator tiles per wave, rescaled by
 //           the per-row online-softmax factor
+// The next tile's global loads are issued one tile ahead into registers, the
+// workgroup's slice of the block table sits in LDS, and single-query steps let
+// the waves that share a row tile split the latent dims (and, for small
+// batches, slice the keys over workgroups with a merge kernel).
 // Scores, softmax statistics and accumulators are f32; the sink enters the
 // denominator at the end.  Window and causality are applied per element from
 // the row's position.  Shapes are compile-time (rank/16, (rank+rot)/32) for a
@@ -59,10 +63,15 @@ __global__ __launch_bounds__(LM_THREADS) void latent_attn_mfma_kernel(
   constexpr int D = KS * 32;
   constexpr int KROW = D + LM_KPAD;
   constexpr int NTW = NT / DS;     // accumulator tiles per wave
+  // Double-buffered images (stage tile i+1 under tile i's products, two
+  // barriers per tile) measured SLOWER than single buffers: the doubled LDS
+  // halves the workgroups per CU, and residency is what hides the latencies.
+  constexpr bool DB = false;
+  constexpr int IMG = LM_KT * KROW + RANK * LM_VROW;   // one K image + one V^T image
   extern __shared__ char lds_raw[];
   bf16* k_img = reinterpret_cast<bf16*>(lds_raw);   // [32][KROW]
   bf16* v_img = k_img + LM_KT * KROW;               // [RANK][LM_VROW]
-  int* bt_s = reinterpret_cast<int*>(v_img + RANK * LM_VROW);   // [LM_BT_MAX]
+  int* bt_s = reinterpret_cast<int*>(k_img + (DB ? 2 : 1) * IMG);   // [LM_BT_MAX]
 
   const int seq = blockIdx.y;
   int q0, nq;
@@ -171,38 +180,38 @@ __global__ __launch_bounds__(LM_THREADS) void latent_attn_mfma_kernel(
       }
     }
   };
-  if (kstart < kend) fetch(kstart);
-
-  for (int base = kstart; base < kend; base += LM_KT) {
-    __syncthreads();   // readers of the previous tile's images are done
+  // pieces of one tile's work; `kb` / `vb` pick the image buffers
+  auto write_k = [&](bf16* kb) {
 #pragma unroll
     for (int i = 0; i < CPT; ++i) {
       const int c = tid + i * LM_THREADS;
       if (c < LM_KT * CPR) {
         const int key = c / CPR, ch = c - key * CPR;
-        *reinterpret_cast<bf16x8_t*>(k_img + key * KROW + ch * 8) = pre[i];
+        *reinterpret_cast<bf16x8_t*>(kb + key * KROW + ch * 8) = pre[i];
       }
     }
-    if (base + LM_KT < kend) fetch(base + LM_KT);
-    __syncthreads();
-    // latent part once more, transposed, keys in contraction-slot order
+  };
+  // latent part once more, transposed, keys in contraction-slot order
+  auto transpose = [&](const bf16* kb, bf16* vb) {
     for (int c = tid; c < LM_KT * (RANK / 8); c += LM_THREADS) {
       const int key = c & 31, ch = c >> 5;
-      const bf16x8_t v = *reinterpret_cast<const bf16x8_t*>(k_img + key * KROW + ch * 8);
+      const bf16x8_t v = *reinterpret_cast<const bf16x8_t*>(kb + key * KROW + ch * 8);
       const int slot = ((key & 15) >> 2) * 8 + (key >> 4) * 4 + (key & 3);
-      short* dst = reinterpret_cast<short*>(v_img) + (ch * 8) * LM_VROW + slot;
+      short* dst = reinterpret_cast<short*>(vb) + (ch * 8) * LM_VROW + slot;
 #pragma unroll
       for (int u = 0; u < 8; ++u) dst[u * LM_VROW] = v[u];
     }
-
+  };
+  bf16x8_t pb;   // this tile's probabilities, B operand of the value product
+  auto scores = [&](const bf16* kb, int base) {
     f32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
     if (wave_active) {
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
         const bf16x8_t a0 = *reinterpret_cast<const bf16x8_t*>(
-            k_img + n * KROW + ks * 32 + g * 8);
+            kb + n * KROW + ks * 32 + g * 8);
         const bf16x8_t a1 = *reinterpret_cast<const bf16x8_t*>(
-            k_img + (16 + n) * KROW + ks * 32 + g * 8);
+            kb + (16 + n) * KROW + ks * 32 + g * 8);
         s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, qf[ks], s0, 0, 0, 0);
         s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, qf[ks], s1, 0, 0, 0);
       }
@@ -222,7 +231,6 @@ __global__ __launch_bounds__(LM_THREADS) void latent_attn_mfma_kernel(
     const float m_new = fmaxf(m_run, mx);
     const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
     const float alpha = (m_run == -INFINITY) ? 0.f : __expf(m_run - m_safe);
-    bf16x8_t pb;
     float ps = 0.f;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -236,14 +244,55 @@ __global__ __launch_bounds__(LM_THREADS) void latent_attn_mfma_kernel(
     for (int i = 0; i < NTW; ++i) {
       acc[i][0] *= alpha; acc[i][1] *= alpha; acc[i][2] *= alpha; acc[i][3] *= alpha;
     }
-    __syncthreads();   // V^T image complete
+  };
+  auto values = [&](const bf16* vb) {
     if (wave_active) {
 #pragma unroll
       for (int dt = 0; dt < NTW; ++dt) {
         const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(
-            v_img + ((dp * NTW + dt) * 16 + n) * LM_VROW + g * 8);
+            vb + ((dp * NTW + dt) * 16 + n) * LM_VROW + g * 8);
         acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb, acc[dt], 0, 0, 0);
       }
+    }
+  };
+
+  if (DB) {
+    // Two image buffers: tile i+1 is staged (K image written, latent part
+    // transposed) while tile i is scored and summed — two barriers per tile,
+    // and the staging LDS traffic fills the gaps between dependent MFMAs.
+    bf16* kbuf[2] = {k_img, k_img + IMG};
+    bf16* vbuf[2] = {v_img, v_img + IMG};
+    if (kstart < kend) {
+      fetch(kstart);
+      write_k(kbuf[0]);
+      if (kstart + LM_KT < kend) fetch(kstart + LM_KT);
+      __syncthreads();
+      transpose(kbuf[0], vbuf[0]);
+    }
+    int cur = 0;
+    for (int base = kstart; base < kend; base += LM_KT, cur ^= 1) {
+      const bool has_next = base + LM_KT < kend;
+      __syncthreads();   // images of `cur` complete; nobody reads the other pair
+      if (has_next) {
+        write_k(kbuf[cur ^ 1]);
+        if (base + 2 * LM_KT < kend) fetch(base + 2 * LM_KT);
+      }
+      scores(kbuf[cur], base);
+      __syncthreads();   // next K image complete
+      if (has_next) transpose(kbuf[cur ^ 1], vbuf[cur ^ 1]);
+      values(vbuf[cur]);
+    }
+  } else {
+    if (kstart < kend) fetch(kstart);
+    for (int base = kstart; base < kend; base += LM_KT) {
+      __syncthreads();   // readers of the previous tile's images are done
+      write_k(k_img);
+      if (base + LM_KT < kend) fetch(base + LM_KT);
+      __syncthreads();
+      transpose(k_img, v_img);
+      scores(k_img, base);
+      __syncthreads();   // V^T image complete
+      values(v_img);
     }
   }
 
@@ -318,7 +367,8 @@ __global__ void latent_attn_merge_kernel(bf16* __restrict__ out, long o_st, long
 // (slice, head) written and read again, so they are only used to give every CU
 // a workgroup when the batch alone does not.
 int latent_decode_num_splits(int nseq, int heads, int max_keys) {
-  const int groups = (heads + LM_ROWS - 1) / LM_ROWS;
+  const int cap = heads <= 16 ? 16 : (heads <= 32 ? 32 : LM_ROWS);
+  const int groups = (heads + cap - 1) / cap;
   const int tiles = (max_keys + LM_KT - 1) / LM_KT;
   // the dim-split variants (<= 32 heads) fit two workgroups per CU
   const int target = heads <= 32 ? 512 : 256;
@@ -351,7 +401,8 @@ static void launch_one(bf16* out, long o_st, long o_sh, const bf16* q_lat,
                        int max_q, int heads, int block_size, int nsplit,
                        float* part_acc, float* part_ml, hipStream_t stream) {
   constexpr int RANK = NT * 16, D = KS * 32;
-  const size_t smem = sizeof(bf16) * (LM_KT * (D + LM_KPAD) + RANK * LM_VROW) +
+  const size_t smem = sizeof(bf16) * (LM_KT * (D + LM_KPAD) + RANK * LM_VROW) *
+                          1 +
                       sizeof(int) * LM_BT_MAX;
   static bool configured = false;
   if (!configured) {
@@ -359,8 +410,9 @@ static void launch_one(bf16* out, long o_st, long o_sh, const bf16* q_lat,
                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     configured = true;
   }
-  const int hpb = heads < LM_ROWS ? heads : LM_ROWS;
-  const int tq = LM_ROWS / hpb;
+  const int rows_cap = LM_ROWS / DS;   // DS waves share a row tile
+  const int hpb = heads < rows_cap ? heads : rows_cap;
+  const int tq = rows_cap / hpb;
   dim3 grid(nsplit > 1 ? nsplit : (max_q + tq - 1) / tq, nseq, (heads + hpb - 1) / hpb);
   latent_attn_mfma_kernel<NT, KS, DS><<<grid, LM_THREADS, smem, stream>>>(
       out, o_st, o_sh, q_lat, ql_st, ql_sh, q_rot, qr_st, qr_sh, cache,
@@ -384,6 +436,10 @@ void launch_latent_attn_mfma(bf16* out, long o_st, long o_sh, const bf16* q_lat,
                              float* part_ml, hipStream_t stream) {
   const int nt = rank / 16, ks = (rank + rot) / 32;
   // one query per sequence and at most one 16-row tile of heads
+  // single queries: as many waves per row tile as the head count leaves free.
+  // (Prompt portions keep four row tiles: splitting dims there — 32 rows per
+  // workgroup, two workgroups per CU at rank 512 — measured 25% slower, the
+  // doubled staging and score work outweighs the residency.)
   const int dim_split = (qsl != nullptr || heads > 32) ? 1 : (heads <= 16 ? 4 : 2);
 #define X(A, B)                                                               \
   if (nt == A && ks == B) {                                                   \
