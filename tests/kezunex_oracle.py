@@ -1,0 +1,238 @@
+"""Plain, slow float64 implementation of the Kezunex design, written from its
+equations: one function per mechanism, whole sequences only, no cache, no
+batching, token-by-token recurrences.  It shares no code with the package and
+is the yardstick for tests/test_kezunex.py.
+
+Notation: h is a sublayer's input [T, width]; weights are stored [out, in]
+and applied as W h; positions count from 0.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+
+F64 = torch.float64
+
+
+def _w(weights, name):
+    return weights[name].to(F64)
+
+
+def lin(w, x, b=None):
+    y = x @ w.T
+    return y if b is None else y + b
+
+
+def gelu_tanh(z):
+    return 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3)))
+
+
+def silu(z):
+    return z * torch.sigmoid(z)
+
+
+def softplus(z):
+    return torch.where(z > 30.0, z, torch.log1p(torch.exp(torch.clamp(z, max=30.0))))
+
+
+def rms_unit(x, eps):
+    return x / torch.sqrt((x * x).mean(dim=-1, keepdim=True) + eps)
+
+
+def layer_norm(x, w, eps):
+    mu = x.mean(dim=-1, keepdim=True)
+    d = x - mu
+    var = (d * d).mean(dim=-1, keepdim=True)
+    return d / torch.sqrt(var + eps) * w
+
+
+def causal_conv(u, w, b):
+    """u [T, C]; w [C, taps] with the last column on the current token; zeros
+    before the start."""
+    t, c = u.shape
+    taps = w.shape[1]
+    out = torch.zeros_like(u)
+    for j in range(taps):
+        shift = taps - 1 - j
+        if shift >= t:
+            continue
+        out[shift:] += u[: t - shift] * w[:, j]
+    return out + b
+
+
+# ---------------------------------------------------------------------------
+# mixers
+# ---------------------------------------------------------------------------
+
+def softmax_attention(h, weights, p, m, eps):
+    """Grouped-query softmax attention, per-head RMS norm on q and k, no
+    rotation, a position-dependent query temperature, causal."""
+    t = h.shape[0]
+    nh, ng, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+    q = lin(_w(weights, p + "q"), h).view(t, nh, d)
+    k = lin(_w(weights, p + "k"), h).view(t, ng, d)
+    v = lin(_w(weights, p + "v"), h).view(t, ng, dv)
+    q = rms_unit(q, eps) * _w(weights, p + "q.norm")
+    k = rms_unit(k, eps) * _w(weights, p + "k.norm")
+    qt = m.get("q_temp")
+    if qt:
+        pos = torch.arange(t, dtype=F64)
+        temp = 1.0 + qt["coef"] * torch.log(torch.floor((pos + 1.0) / qt["every"]) + 1.0)
+        q = q * temp.view(t, 1, 1)
+    out = torch.zeros(t, nh, dv, dtype=F64)
+    per = nh // ng
+    for hd in range(nh):
+        g = hd // per
+        s = (q[:, hd] @ k[:, g].T) * m["scale"]
+        mask = torch.ones(t, t, dtype=torch.bool).tril()
+        s = s.masked_fill(~mask, float("-inf"))
+        out[:, hd] = torch.softmax(s, dim=-1) @ v[:, g]
+    return lin(_w(weights, p + "o"), out.reshape(t, nh * dv))
+
+
+def ssd(h, weights, p, m, eps):
+    """State-space-duality recurrence with a short convolution in front and a
+    gated grouped RMS norm behind."""
+    t = h.shape[0]
+    nh, dv, n, g = m["heads"], m["vdim"], m["state"], m["groups"]
+    inner = nh * dv
+    zxbcdt = lin(_w(weights, p + "in"), h)
+    z = zxbcdt[:, :inner]
+    xbc = zxbcdt[:, inner:2 * inner + 2 * g * n]
+    dt = zxbcdt[:, 2 * inner + 2 * g * n:]
+    xbc = silu(causal_conv(xbc, _w(weights, p + "conv"), _w(weights, p + "conv.b")))
+    x = xbc[:, :inner].view(t, nh, dv)
+    bmat = xbc[:, inner:inner + g * n].view(t, g, n)
+    cmat = xbc[:, inner + g * n:].view(t, g, n)
+    dt = softplus(dt + _w(weights, p + "dt_bias"))
+    a = torch.exp(_w(weights, p + "A_log"))
+    dskip = _w(weights, p + "D")
+    per = nh // g
+    y = torch.zeros(t, nh, dv, dtype=F64)
+    for hd in range(nh):
+        grp = hd // per
+        s = torch.zeros(n, dv, dtype=F64)
+        for i in range(t):
+            s = math.exp(-a[hd].item() * dt[i, hd].item()) * s \
+                + dt[i, hd] * torch.outer(bmat[i, grp], x[i, hd])
+            y[i, hd] = s.T @ cmat[i, grp] + dskip[hd] * x[i, hd]
+    y = y.reshape(t, inner) * silu(z)
+    ng = m["norm_groups"]
+    y = rms_unit(y.view(t, ng, inner // ng), eps).reshape(t, inner) * _w(weights, p + "norm")
+    return lin(_w(weights, p + "o"), y)
+
+
+def parallel_mixer(h, weights, p, m, eps):
+    left = softmax_attention(h, weights, p + "left.", m["left"], eps)
+    right = ssd(h, weights, p + "right.", m["right"], eps)
+    return m["left_scale"] * left + m["right_scale"] * right
+
+
+def rglru(h, weights, p, m, eps):
+    """Recurrent block with a real-gated linear recurrent unit."""
+    t = h.shape[0]
+    width, nb = m["width"], m["blocks"]
+    y = gelu_tanh(lin(_w(weights, p + "y"), h, _w(weights, p + "y.b")))
+    u = causal_conv(lin(_w(weights, p + "x"), h, _w(weights, p + "x.b")),
+                    _w(weights, p + "conv"), _w(weights, p + "conv.b"))
+    ub = u.view(t, nb, width // nb)
+    ra, rab = _w(weights, p + "ra"), _w(weights, p + "ra.b")
+    ri, rib = _w(weights, p + "ri"), _w(weights, p + "ri.b")
+    r = torch.sigmoid(torch.einsum("boi,tbi->tbo", ra, ub) + rab).reshape(t, width)
+    gate = torch.sigmoid(torch.einsum("boi,tbi->tbo", ri, ub) + rib).reshape(t, width)
+    log_a = -8.0 * r * softplus(_w(weights, p + "lam"))
+    a = torch.exp(log_a)
+    s = torch.zeros(width, dtype=F64)
+    out = torch.zeros(t, width, dtype=F64)
+    for i in range(t):
+        s = a[i] * s + torch.sqrt(1.0 - a[i] ** 2) * gate[i] * u[i]
+        out[i] = s
+    return lin(_w(weights, p + "o"), out * y)
+
+
+def mlstm(h, weights, p, m, eps):
+    """Matrix memory with exponential gating and a running maximum that
+    starts at 0."""
+    t = h.shape[0]
+    nh, d, dv, cap = m["heads"], m["dim"], m["vdim"], m["gate_cap"]
+    q = (lin(_w(weights, p + "q"), h) * d ** -0.5).view(t, nh, d)
+    k = lin(_w(weights, p + "k"), h).view(t, nh, d)
+    v = lin(_w(weights, p + "v"), h).view(t, nh, dv)
+    ig = cap * torch.tanh(lin(_w(weights, p + "i"), h, _w(weights, p + "i.b")) / cap)
+    fg = torch.nn.functional.logsigmoid(
+        cap * torch.tanh(lin(_w(weights, p + "f"), h, _w(weights, p + "f.b")) / cap))
+    o = torch.zeros(t, nh, dv, dtype=F64)
+    for hd in range(nh):
+        s = torch.zeros(d, dv, dtype=F64)
+        n = torch.zeros(d, dtype=F64)
+        mx = 0.0
+        for i in range(t):
+            f, g = fg[i, hd].item(), ig[i, hd].item()
+            m_new = max(f + mx, g)
+            s = math.exp(f + mx - m_new) * s + math.exp(g - m_new) * torch.outer(k[i, hd], v[i, hd])
+            n = math.exp(f + mx - m_new) * n + math.exp(g - m_new) * k[i, hd]
+            mx = m_new
+            den = max(abs(float(n @ q[i, hd])), math.exp(-mx)) + 1e-6
+            o[i, hd] = (s.T @ q[i, hd]) / den
+    o = rms_unit(o, eps).reshape(t, nh * dv) * _w(weights, p + "norm")
+    o = o * torch.sigmoid(lin(_w(weights, p + "g"), h))
+    return lin(_w(weights, p + "o"), o)
+
+
+MIXERS = {"parallel": parallel_mixer, "rglru": rglru, "mlstm": mlstm}
+
+
+def dense_ff(h, weights, p):
+    return lin(_w(weights, p + "down"),
+               gelu_tanh(lin(_w(weights, p + "gate"), h)) * lin(_w(weights, p + "up"), h))
+
+
+# ---------------------------------------------------------------------------
+# whole model
+# ---------------------------------------------------------------------------
+
+def layer_schedule(cfg):
+    """[(layer index, pass number or None, first of its pass)] in run order."""
+    n = len(cfg["layers"])
+    loop = cfg.get("loop")
+    if not loop:
+        return [(i, None, False) for i in range(n)]
+    a, b, times = loop["start"], loop["stop"], loop["times"]
+    runs = [(i, None, False) for i in range(a)]
+    for t in range(times):
+        runs += [(i, t, i == a) for i in range(a, b)]
+    runs += [(i, None, False) for i in range(b, n)]
+    return runs
+
+
+def forward(cfg, weights, tokens, return_layers=False):
+    """Logits [T, vocab] (f64) for one whole sequence; optionally also the
+    residual stream after every layer run."""
+    eps = cfg["norm"]["eps"]
+    ids = torch.as_tensor(tokens, dtype=torch.long)
+    emb = _w(weights, "embed")
+    x0 = emb[ids] * cfg["embedding"]["scale"]
+    x = x0.clone()
+    streams = []
+    for i, t, first in layer_schedule(cfg):
+        if first:
+            if t > 0:
+                x = x + x0
+            x = x + _w(weights, "loop.step")[t]
+        spec = cfg["layers"][i]
+        p = f"l{i}."
+        h = layer_norm(x, _w(weights, p + "norm1"), eps)
+        y = MIXERS[spec["type"]](h, weights, p + "mix.", spec["mixer"], eps)
+        x = x + layer_norm(y, _w(weights, p + "norm1b"), eps) * _w(weights, p + "ls1")
+        if spec.get("mlp") is not None:
+            h = layer_norm(x, _w(weights, p + "norm2"), eps)
+            y = dense_ff(h, weights, p + "mlp.")
+            x = x + layer_norm(y, _w(weights, p + "norm2b"), eps) * _w(weights, p + "ls2")
+        streams.append(x.clone())
+    x = layer_norm(x, _w(weights, "final.norm"), eps)
+    logits = x @ emb.T
+    if return_layers:
+        return logits, torch.stack(streams)
+    return logits

@@ -22,4 +22,21 @@ def get_model(cfg: ModelConfig):
         from .dolodra import DolodraForCausalLM
 
         return DolodraForCausalLM(cfg)
+    if cfg.architecture == "kezunex":
+        from .kezunex import KezunexForCausalLM
+
+        return KezunexForCausalLM(cfg)
     raise ValueError(f"Unsupported architecture: {cfg.architecture}")
+
+
+def native_extensions(cfg: ModelConfig) -> list[str]:
+    """Names of the compiled extensions (kernels/build.py) whose ops the
+    model's forward reaches on a GPU — what a fresh checkout has to build
+    before it can serve this model."""
+    if cfg.architecture == "dolodra":
+        return ["_C_seq"]
+    if cfg.architecture == "kezunex":
+        from .kezunex import native_extensions as kz
+
+        return kz(cfg)
+    return ["_C"]

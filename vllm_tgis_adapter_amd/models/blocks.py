@@ -13,6 +13,22 @@ that another design can assemble them differently:
 - ``DenseMLP``          down(act(up(h))) with the tanh-form GELU
 - ``TokenSideInput``    gated per-layer token embedding added to the stream
                         through its own RMS norm
+- ``StreamLayerNorm``   bias-free layer norm of the f32 stream
+- ``GatedDenseMLP``     down(act(gate(h)) * up(h)) with the tanh-form GELU
+- ``QKNormAttention``   grouped-query softmax attention over the paged cache,
+                        per-head RMS norm on queries and keys, no rotation, an
+                        optional position-dependent query temperature; the
+                        value size may differ from the query/key size
+- ``SSDMixer``          state-space-duality recurrence (short convolution,
+                        per-head scalar decay, gated grouped RMS norm)
+- ``RGLRUMixer``        recurrent block with a real-gated linear recurrent unit
+- ``MLSTMMixer``        matrix memory with exponential gating
+- ``ParallelMixer``     two mixers reading the same input through one merged
+                        projection, their outputs mixed with fixed scales
+
+The recurrent mixers keep their state (f32) and the last inputs of their short
+convolutions in per-sequence slots; a sequence that starts in a step starts
+from zero state whatever its slot held before.
 
 The stream itself, norms, rotation angles, attention scores and softmax are
 f32 whatever the compute dtype is; projections run in the compute dtype.
@@ -201,3 +217,374 @@ class TokenSideInput(nn.Module):
         if next_norm is not None:
             nn_ = (next_norm.weight, next_norm.eps, next_norm.weight_offset, next_norm.dtype)
         return ops.stream_add_rms_norm(x, y, self.norm, self.eps, self.mult, nn_)
+
+
+# ---------------------------------------------------------------------------
+# Layer-norm stream blocks, softmax attention with query/key norm, recurrent
+# mixers.  Mixers share one shape: ``in_rows`` rows of an input projection
+# (own weight, or a slice of a merged one when ``own_in`` is False), ``mix``
+# from the projected rows to the rows that ``o_weight`` maps back to the
+# width, and ``cache_shapes`` naming what they keep per cache block / slot.
+# ---------------------------------------------------------------------------
+
+
+def _randn_param(shape, dtype, std: float = 0.02) -> nn.Parameter:
+    return nn.Parameter(torch.empty(*shape, dtype=dtype).normal_(0.0, std),
+                        requires_grad=False)
+
+
+class StreamLayerNorm(nn.Module):
+    """f32 stream -> compute dtype: (x - mean) / sqrt(var + eps) * w, no bias."""
+
+    def __init__(self, width: int, eps: float, dtype: torch.dtype):
+        super().__init__()
+        self.eps = eps
+        self.dtype = dtype
+        self.weight = _f32_param(width, fill=1.0)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return ops.layer_norm_stream(x, self.weight, self.eps, self.dtype)
+
+    def as_next(self):
+        return (self.weight, self.eps, self.dtype)
+
+
+class GatedDenseMLP(nn.Module):
+    """down(gelu_tanh(gate h) * (up h)); gate and up are one merged product."""
+
+    def __init__(self, width: int, ff: int, dtype: torch.dtype):
+        super().__init__()
+        if get_tp_world_size() != 1:
+            raise ValueError("GatedDenseMLP is not sharded; run it with one rank")
+        self.ff = ff
+        self.gate_up = _randn_param((2 * ff, width), dtype)
+        self.down = _randn_param((width, ff), dtype)
+
+    def load(self, gate, up, down) -> None:
+        self.gate_up.data[:self.ff].copy_(gate.to(self.gate_up.dtype))
+        self.gate_up.data[self.ff:].copy_(up.to(self.gate_up.dtype))
+        self.down.data.copy_(down.to(self.down.dtype))
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        gu = ops.linear(h, self.gate_up)
+        a = ops.gelu_tanh(gu[:, :self.ff].contiguous(), mul=gu[:, self.ff:])
+        return ops.linear(a, self.down)
+
+
+class _Mixer(nn.Module):
+    """Common shape of the mixers below (see the section comment)."""
+
+    in_rows: int
+    out_rows: int
+    has_in_bias = False
+
+    def _alloc(self, width: int, own_in: bool, dtype: torch.dtype) -> None:
+        if get_tp_world_size() != 1:
+            raise ValueError(f"{type(self).__name__} is not sharded; run it with one rank")
+        self.width = width
+        self.dtype = dtype
+        self.in_weight = _randn_param((self.in_rows, width), dtype) if own_in else None
+        self.in_bias = (nn.Parameter(torch.zeros(self.in_rows, dtype=dtype), requires_grad=False)
+                        if own_in and self.has_in_bias else None)
+        self.o_weight = _randn_param((width, self.out_rows), dtype)
+
+    def project(self, h: torch.Tensor) -> torch.Tensor:
+        return ops.linear(h, self.in_weight, self.in_bias)
+
+    def forward(self, h, positions, cache, meta: AttnMetadata) -> torch.Tensor:
+        return ops.linear(self.mix(self.project(h), positions, cache, meta), self.o_weight)
+
+    def load_in(self, weight: torch.Tensor, bias, tensors: dict) -> None:
+        raise NotImplementedError
+
+    def load(self, tensors: dict) -> None:
+        """tensors: this mixer's checkpoint tensors by their short names."""
+        self.load_in(self.in_weight.data, None if self.in_bias is None else self.in_bias.data,
+                     tensors)
+        self.o_weight.data.copy_(tensors["o"].to(self.dtype))
+        self.load_rest(tensors)
+
+    def load_rest(self, tensors: dict) -> None:
+        pass
+
+    # what the mixer keeps: {name: (kind, shape-per-block-or-slot, dtype)} with
+    # kind "paged" (per cache block) or "slot" (per sequence)
+    def cache_shapes(self, block_size: int) -> list:
+        return []
+
+
+class QKNormAttention(_Mixer):
+    """Causal grouped-query softmax attention.  q, k are RMS-normed per head
+    with a weight shared by all heads (plain weight); positions enter only
+    through the optional query temperature 1 + coef * ln(floor((p + 1) /
+    every) + 1); score = q . k * scale.  Projected rows: [q | k | v]."""
+
+    def __init__(self, width: int, *, heads: int, kv_heads: int, dim: int, vdim: int,
+                 scale: float, eps: float, temp_coef: float = 0.0, temp_every: int = 0,
+                 own_in: bool = True, dtype: torch.dtype = torch.bfloat16):
+        super().__init__()
+        if heads % kv_heads:
+            raise ValueError("heads must be a multiple of kv_heads")
+        self.heads, self.kv_heads, self.dim, self.vdim = heads, kv_heads, dim, vdim
+        self.scale, self.eps = scale, eps
+        self.temp_coef, self.temp_every = temp_coef, temp_every
+        self.in_rows = heads * dim + kv_heads * (dim + vdim)
+        self.out_rows = heads * vdim
+        self._alloc(width, own_in, dtype)
+        self.q_norm = _f32_param(dim, fill=1.0)
+        self.k_norm = _f32_param(dim, fill=1.0)
+
+    def load_in(self, weight, bias, t) -> None:
+        a = self.heads * self.dim
+        b = a + self.kv_heads * self.dim
+        weight[:a].copy_(t["q"].to(weight.dtype))
+        weight[a:b].copy_(t["k"].to(weight.dtype))
+        weight[b:].copy_(t["v"].to(weight.dtype))
+
+    def load_rest(self, t) -> None:
+        self.q_norm.data.copy_(t["q.norm"].float())
+        self.k_norm.data.copy_(t["k.norm"].float())
+
+    def cache_shapes(self, block_size: int) -> list:
+        return [("paged", (block_size, self.kv_heads, self.dim), self.dtype),
+                ("paged", (block_size, self.kv_heads, self.vdim), self.dtype)]
+
+    def mix(self, proj, positions, cache, meta: AttnMetadata) -> torch.Tensor:
+        t = proj.shape[0]
+        nh, ng, d, dv = self.heads, self.kv_heads, self.dim, self.vdim
+        a = nh * d
+        b = a + ng * d
+        k_cache, v_cache = cache
+        q = ops.qk_norm_cache_write(
+            proj[:, :a].view(t, nh, d), proj[:, a:b].view(t, ng, d),
+            proj[:, b:].view(t, ng, dv), self.q_norm, self.k_norm, self.eps,
+            positions, self.temp_coef, self.temp_every, k_cache, v_cache,
+            meta.slot_mapping)
+        out = torch.empty((t, nh, dv), dtype=proj.dtype, device=proj.device)
+        npt = meta.num_prefill_tokens
+        if npt:
+            ops.gqa_attention_prefill(
+                q[:npt], k_cache, v_cache, meta.prefill_block_tables,
+                meta.prefill_query_start_loc, meta.prefill_seq_lens, self.scale,
+                meta.max_prefill_query_len, out=out[:npt])
+        if meta.num_decode_seqs:
+            ops.gqa_attention_decode(
+                q[npt:], k_cache, v_cache, meta.decode_block_tables,
+                meta.decode_seq_lens, self.scale, out=out[npt:])
+        return out.view(t, nh * dv)
+
+
+class SSDMixer(_Mixer):
+    """State-space-duality mixer.  Projected rows: [z | x | B | C | dt] with
+    inner = heads * vdim, B and C of groups * state each.  x, B, C pass a short
+    causal convolution with bias and silu; dt = softplus(dt + dt_bias); per
+    head S_t = exp(-exp(A_log) dt) S_(t-1) + dt B_t x_t^T, y_t = S_t^T C_t + D
+    x_t; y * silu(z) is RMS-normed in ``norm_groups`` parts, times a weight."""
+
+    def __init__(self, width: int, *, heads: int, vdim: int, state: int, groups: int,
+                 taps: int, norm_groups: int, eps: float, own_in: bool = True,
+                 dtype: torch.dtype = torch.bfloat16):
+        super().__init__()
+        if heads % groups or (heads * vdim) % norm_groups:
+            raise ValueError("heads must divide by groups, inner size by norm_groups")
+        self.heads, self.vdim, self.nstate, self.groups = heads, vdim, state, groups
+        self.taps, self.norm_groups, self.eps = taps, norm_groups, eps
+        self.inner = heads * vdim
+        self.conv_ch = self.inner + 2 * groups * state
+        self.in_rows = self.inner + self.conv_ch + heads
+        self.out_rows = self.inner
+        self._alloc(width, own_in, dtype)
+        self.conv_weight = nn.Parameter(
+            torch.empty(self.conv_ch, taps, dtype=torch.float32).normal_(0.0, 0.2),
+            requires_grad=False)
+        self.conv_bias = _f32_param(self.conv_ch)
+        # step sizes around 0.01..0.1 and decays A in 1..16 for random weights
+        self.dt_bias = nn.Parameter(torch.empty(heads).uniform_(-4.6, -2.2), requires_grad=False)
+        self.a_log = nn.Parameter(torch.empty(heads).uniform_(0.0, 2.77), requires_grad=False)
+        self.d_skip = _f32_param(heads, fill=1.0)
+        self.norm = _f32_param(self.inner, fill=1.0)
+
+    def load_in(self, weight, bias, t) -> None:
+        weight.copy_(t["in"].to(weight.dtype))
+
+    def load_rest(self, t) -> None:
+        self.conv_weight.data.copy_(t["conv"].float())
+        self.conv_bias.data.copy_(t["conv.b"].float())
+        self.dt_bias.data.copy_(t["dt_bias"].float())
+        self.a_log.data.copy_(t["A_log"].float())
+        self.d_skip.data.copy_(t["D"].float())
+        self.norm.data.copy_(t["norm"].float())
+
+    def cache_shapes(self, block_size: int) -> list:
+        return [("slot", (max(self.taps - 1, 0), self.conv_ch), self.dtype),
+                ("slot", (self.heads, self.nstate, self.vdim), torch.float32)]
+
+    def mix(self, proj, positions, cache, meta: AttnMetadata) -> torch.Tensor:
+        conv_state, ssm_state = cache
+        inner = self.inner
+        z = proj[:, :inner]
+        xbc = ops.causal_conv_state(
+            proj[:, inner:inner + self.conv_ch], self.conv_weight, conv_state,
+            meta.seq_start_loc, meta.seq_lens, meta.state_slots, add_input=False,
+            bias=self.conv_bias, act="silu")
+        y = ops.ssd_scan(xbc, proj[:, inner + self.conv_ch:], self.dt_bias, self.a_log,
+                         self.d_skip, ssm_state, meta.seq_start_loc, meta.seq_lens,
+                         meta.state_slots, self.heads, self.vdim, self.nstate, self.groups)
+        return ops.gated_group_norm(y, z, self.norm, self.norm_groups, self.eps,
+                                    gate_first=True, out_dtype=self.dtype)
+
+
+class RGLRUMixer(_Mixer):
+    """Recurrent block: y = gelu_tanh(W_y h + b), u = conv(W_x h + b) (short
+    causal convolution with bias, no activation); per block of channels r =
+    sigmoid(R_a u + b), i = sigmoid(R_i u + b); a = exp(-c r softplus(lam)),
+    S_t = a S_(t-1) + sqrt(1 - a^2) i u; output rows S * y.  Projected rows:
+    [y | x]."""
+
+    has_in_bias = True
+
+    def __init__(self, width: int, *, rec_width: int, blocks: int, taps: int,
+                 gate_c: float = 8.0, own_in: bool = True,
+                 dtype: torch.dtype = torch.bfloat16):
+        super().__init__()
+        if rec_width % blocks:
+            raise ValueError("recurrent width must divide by blocks")
+        self.rec_width, self.blocks, self.taps, self.gate_c = rec_width, blocks, taps, gate_c
+        self.in_rows = 2 * rec_width
+        self.out_rows = rec_width
+        self._alloc(width, own_in, dtype)
+        bw = rec_width // blocks
+        self.conv_weight = nn.Parameter(
+            torch.empty(rec_width, taps, dtype=torch.float32).normal_(0.0, 0.2),
+            requires_grad=False)
+        self.conv_bias = _f32_param(rec_width)
+        # stored transposed ([block, in, out]) for the batched product
+        self.ra_t = _randn_param((blocks, bw, bw), dtype, std=bw ** -0.5)
+        self.ri_t = _randn_param((blocks, bw, bw), dtype, std=bw ** -0.5)
+        self.ra_bias = _f32_param(rec_width)
+        self.ri_bias = _f32_param(rec_width)
+        self.lam = nn.Parameter(torch.empty(rec_width).uniform_(-4.0, -1.0), requires_grad=False)
+
+    def load_in(self, weight, bias, t) -> None:
+        w = self.rec_width
+        weight[:w].copy_(t["y"].to(weight.dtype))
+        weight[w:].copy_(t["x"].to(weight.dtype))
+        bias[:w].copy_(t["y.b"].to(bias.dtype))
+        bias[w:].copy_(t["x.b"].to(bias.dtype))
+
+    def load_rest(self, t) -> None:
+        self.conv_weight.data.copy_(t["conv"].float())
+        self.conv_bias.data.copy_(t["conv.b"].float())
+        self.ra_t.data.copy_(t["ra"].transpose(1, 2).to(self.dtype))
+        self.ri_t.data.copy_(t["ri"].transpose(1, 2).to(self.dtype))
+        self.ra_bias.data.copy_(t["ra.b"].float().reshape(-1))
+        self.ri_bias.data.copy_(t["ri.b"].float().reshape(-1))
+        self.lam.data.copy_(t["lam"].float())
+
+    def cache_shapes(self, block_size: int) -> list:
+        return [("slot", (max(self.taps - 1, 0), self.rec_width), self.dtype),
+                ("slot", (self.rec_width,), torch.float32)]
+
+    def mix(self, proj, positions, cache, meta: AttnMetadata) -> torch.Tensor:
+        conv_state, rec_state = cache
+        t, w, nb = proj.shape[0], self.rec_width, self.blocks
+        yb = ops.gelu_tanh(proj[:, :w].contiguous())
+        u = ops.causal_conv_state(
+            proj[:, w:], self.conv_weight, conv_state, meta.seq_start_loc,
+            meta.seq_lens, meta.state_slots, add_input=False, bias=self.conv_bias)
+        ub = u.view(t, nb, w // nb).transpose(0, 1)              # [blocks, T, bw]
+        r_pre = torch.bmm(ub, self.ra_t).transpose(0, 1).reshape(t, w)
+        i_pre = torch.bmm(ub, self.ri_t).transpose(0, 1).reshape(t, w)
+        return ops.rglru_scan(u, r_pre, i_pre, self.ra_bias, self.ri_bias, self.lam,
+                              self.gate_c, yb, rec_state, meta.seq_start_loc,
+                              meta.seq_lens, meta.state_slots)
+
+
+class MLSTMMixer(_Mixer):
+    """Matrix memory with exponential gating.  q = W_q h / sqrt(dim), k, v per
+    head; log input gate i = cap tanh((W_i h + b) / cap), log forget gate f =
+    logsigmoid(cap tanh((W_f h + b) / cap)); running maximum m (0 at the
+    start): m_t = max(f + m, i), S_t = exp(f + m - m_t) S + exp(i - m_t) k v^T, n
+    likewise with k; o = S^T q / (max(|n . q|, exp(-m_t)) + 1e-6); each head's o
+    is RMS-normed, times a weight, times sigmoid(W_g h).  Projected rows:
+    [q | k | v | g | i | f]."""
+
+    def __init__(self, width: int, *, heads: int, dim: int, vdim: int, gate_cap: float,
+                 eps: float, own_in: bool = True, dtype: torch.dtype = torch.bfloat16):
+        super().__init__()
+        self.heads, self.dim, self.vdim = heads, dim, vdim
+        self.gate_cap, self.eps = gate_cap, eps
+        self.in_rows = 2 * heads * dim + 2 * heads * vdim + 2 * heads
+        self.out_rows = heads * vdim
+        self._alloc(width, own_in, dtype)
+        self.i_bias = _f32_param(heads)
+        self.f_bias = _f32_param(heads, fill=3.0)
+        self.norm = _f32_param(heads * vdim, fill=1.0)
+
+    def load_in(self, weight, bias, t) -> None:
+        off = 0
+        for name in ("q", "k", "v", "g", "i", "f"):
+            n = t[name].shape[0]
+            weight[off:off + n].copy_(t[name].to(weight.dtype))
+            off += n
+
+    def load_rest(self, t) -> None:
+        self.i_bias.data.copy_(t["i.b"].float())
+        self.f_bias.data.copy_(t["f.b"].float())
+        self.norm.data.copy_(t["norm"].float())
+
+    def cache_shapes(self, block_size: int) -> list:
+        return [("slot", (self.heads, self.dim, self.vdim), torch.float32),
+                ("slot", (self.heads, self.dim), torch.float32),
+                ("slot", (self.heads,), torch.float32)]
+
+    def mix(self, proj, positions, cache, meta: AttnMetadata) -> torch.Tensor:
+        s_state, n_state, m_state = cache
+        t, nh, d, dv = proj.shape[0], self.heads, self.dim, self.vdim
+        a = nh * d
+        b = 2 * a
+        c = b + nh * dv
+        e = c + nh * dv
+        o = ops.mlstm_scan(
+            proj[:, :a].view(t, nh, d), proj[:, a:b].view(t, nh, d),
+            proj[:, b:c].view(t, nh, dv), proj[:, e:e + nh], proj[:, e + nh:],
+            self.i_bias, self.f_bias, self.gate_cap, d ** -0.5, s_state, n_state,
+            m_state, meta.seq_start_loc, meta.seq_lens, meta.state_slots)
+        return ops.gated_group_norm(o, proj[:, c:e], self.norm, nh, self.eps,
+                                    gate_first=False, out_dtype=self.dtype)
+
+
+class ParallelMixer(nn.Module):
+    """Two mixers side by side on the same input: one merged input projection,
+    result = left_scale * left + right_scale * right.  Returns the two outputs
+    and their scales; the caller's residual kernel forms the sum in f32."""
+
+    def __init__(self, width: int, left: _Mixer, right: _Mixer, left_scale: float,
+                 right_scale: float, dtype: torch.dtype):
+        super().__init__()
+        if left.has_in_bias or right.has_in_bias:
+            raise ValueError("merged projection of mixers with input bias is not supported")
+        self.left, self.right = left, right
+        self.left_scale, self.right_scale = left_scale, right_scale
+        self.in_weight = _randn_param((left.in_rows + right.in_rows, width), dtype)
+
+    def load(self, left_tensors: dict, right_tensors: dict) -> None:
+        n = self.left.in_rows
+        for mod, rows, t in ((self.left, self.in_weight.data[:n], left_tensors),
+                             (self.right, self.in_weight.data[n:], right_tensors)):
+            mod.load_in(rows, None, t)
+            mod.o_weight.data.copy_(t["o"].to(mod.dtype))
+            mod.load_rest(t)
+
+    def cache_shapes(self, block_size: int) -> list:
+        return self.left.cache_shapes(block_size) + self.right.cache_shapes(block_size)
+
+    def forward(self, h, positions, cache, meta: AttnMetadata):
+        proj = ops.linear(h, self.in_weight)
+        n = self.left.in_rows
+        nl = len(self.left.cache_shapes(1))
+        a = ops.linear(self.left.mix(proj[:, :n], positions, cache[:nl], meta),
+                       self.left.o_weight)
+        b = ops.linear(self.right.mix(proj[:, n:], positions, cache[nl:], meta),
+                       self.right.o_weight)
+        return a, b

@@ -430,6 +430,12 @@ def _try_load_seq() -> None:
 _try_load_seq()
 
 
+def reload_native() -> None:
+    """Load extensions that were built after this module was imported."""
+    _try_load_native()
+    _try_load_seq()
+
+
 def has_native_seq() -> bool:
     _try_load_seq()
     return _S is not None
@@ -523,17 +529,23 @@ def softcap(logits: torch.Tensor, cap: float) -> torch.Tensor:
 
 
 def causal_conv_state(h, weight, state, seq_start_loc, seq_lens, state_slots,
-                      add_input: bool = True) -> torch.Tensor:
+                      add_input: bool = True, bias: torch.Tensor | None = None,
+                      act: str | None = None) -> torch.Tensor:
     """Depthwise causal convolution over each sequence's new rows with the
-    last taps-1 inputs carried in ``state[slot]`` (advanced in place)."""
+    last taps-1 inputs carried in ``state[slot]`` (advanced in place).  ``h``
+    may be a column slice of a wider matrix; ``bias`` [W] f32 and ``act``
+    ("silu") are applied to the result."""
+    if act not in (None, "silu"):
+        raise ValueError(f"unknown activation {act!r}")
     if h.numel() and _native_seq(h):
-        out = torch.empty_like(h)
+        out = torch.empty(h.shape, dtype=h.dtype, device=h.device)
         _S.causal_conv_state(out, h, weight, state, seq_start_loc, seq_lens,
-                             state_slots, bool(add_input))
+                             state_slots, bool(add_input), bias,
+                             1 if act == "silu" else 0)
         return out
     return reference.causal_conv_state(
         h, weight, state, seq_start_loc.cpu(), seq_lens.cpu(), state_slots.cpu(),
-        add_input)
+        add_input, bias, act)
 
 
 def rope_partial(x: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor,
@@ -591,3 +603,195 @@ def latent_attention_decode(q_lat, q_rot, cache, block_tables, seq_lens, scale,
         q_lat, q_rot, cache, block_tables.cpu(), qsl, seq_lens.cpu(), scale,
         window, sinks))
     return out
+
+
+# ---------------------------------------------------------------------------
+# Layer norm of the f32 stream, grouped-query softmax attention with per-head
+# query/key norm (any query/key and value size, f32 or bf16), recurrent mixers
+# with per-sequence f32 state.  Same extension as the stream ops.
+# ---------------------------------------------------------------------------
+
+
+def layer_norm_stream(x: torch.Tensor, weight: torch.Tensor, eps: float,
+                      out_dtype: torch.dtype) -> torch.Tensor:
+    """Bias-free layer norm of an f32 stream into the compute dtype."""
+    if x.numel() and _native_seq(x):
+        out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+        _S.layer_norm_stream(out, x, weight, float(eps))
+        return out
+    return reference.layer_norm_stream(x, weight, eps, out_dtype)
+
+
+def stream_add_layer_norm(x: torch.Tensor, a: torch.Tensor, b: torch.Tensor | None,
+                          scale_a: float, scale_b: float, weight: torch.Tensor,
+                          layer_scale: torch.Tensor | None, eps: float,
+                          next_norm=None):
+    """x (f32, in place) += LN(scale_a * a + scale_b * b) * weight * layer_scale.
+
+    ``next_norm`` = (weight, eps, dtype): the layer norm that reads the updated
+    stream next is computed in the same pass and returned."""
+    if x.numel() and _native_seq(x):
+        out = None
+        nw, neps = None, 0.0
+        if next_norm is not None:
+            nw, neps, ndtype = next_norm
+            out = torch.empty(x.shape, dtype=ndtype, device=x.device)
+        _S.stream_add_layer_norm(x, a, b, float(scale_a), float(scale_b), weight,
+                                 layer_scale, float(eps), out, nw, float(neps))
+        return out
+    reference.stream_add_layer_norm(x, a, b, scale_a, scale_b, weight, layer_scale, eps)
+    if next_norm is None:
+        return None
+    nw, neps, ndtype = next_norm
+    return reference.layer_norm_stream(x, nw, neps, ndtype)
+
+
+def stream_add_vec(x: torch.Tensor, other: torch.Tensor | None, vec: torch.Tensor) -> None:
+    """x (f32, in place) += other + vec, vec [width] broadcast over rows."""
+    if x.numel() and _native_seq(x):
+        _S.stream_add_vec(x, other, vec)
+        return
+    reference.stream_add_vec(x, other, vec)
+
+
+def qk_norm_cache_write(q, k, v, q_weight, k_weight, eps, positions, temp_coef,
+                        temp_every, k_cache, v_cache, slot_mapping) -> torch.Tensor:
+    """Per-head RMS norm of q [T, H, dim] and k [T, G, dim] (views into a merged
+    projection are fine), position-dependent query temperature, normed keys and
+    v [T, G, vdim] stored in the paged cache.  Returns contiguous queries."""
+    if q.numel() and _native_seq(q):
+        out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+        _S.qk_norm_cache_write(out, q, k, v, q_weight, k_weight, float(eps),
+                               positions, float(temp_coef), int(temp_every),
+                               k_cache, v_cache, slot_mapping)
+        return out
+    return reference.qk_norm_cache_write(q, k, v, q_weight, k_weight, eps, positions,
+                                         temp_coef, temp_every, k_cache, v_cache,
+                                         slot_mapping)
+
+
+def _matrix_core_attention_fits(q: torch.Tensor, k_cache: torch.Tensor,
+                                v_cache: torch.Tensor) -> bool:
+    """The llama-class MFMA kernels of ``_C`` take bf16, equal query/key and
+    value sizes of 64 or 128 and up to 8 query heads per key head."""
+    if _C is None or _FORCE_REFERENCE or q.dtype != torch.bfloat16:
+        return False
+    d = q.shape[-1]
+    group = q.shape[1] // k_cache.shape[2]
+    return (d in (64, 128) and v_cache.shape[-1] == d and 1 <= group <= 8
+            and q.shape[1] == group * k_cache.shape[2])
+
+
+def attention_uses_matrix_cores(dtype: torch.dtype, heads: int, kv_heads: int,
+                                dim: int, vdim: int) -> bool:
+    """Shape test of the above without tensors (which extensions a model needs)."""
+    return (dtype == torch.bfloat16 and dim == vdim and dim in (64, 128)
+            and heads % kv_heads == 0 and 1 <= heads // kv_heads <= 8)
+
+
+def gqa_attention_prefill(q, k_cache, v_cache, block_tables, query_start_loc,
+                          seq_lens, scale, max_query_len, out: torch.Tensor) -> torch.Tensor:
+    """Causal grouped-query softmax attention of query chunks (the tail rows
+    of each sequence) over the paged cache; q [T, H, dim], out [T, H, vdim].
+    bf16 shapes the MFMA kernels take run there, everything else (f32, other
+    sizes, value size unlike the key size) on the any-shape kernel."""
+    if q.numel() and _native_seq(q):
+        if _matrix_core_attention_fits(q, k_cache, v_cache):
+            tmp = torch.empty_like(q)
+            _C.paged_attention_prefill(tmp, q, k_cache, v_cache, block_tables,
+                                       query_start_loc, seq_lens, float(scale),
+                                       int(max_query_len))
+            out.copy_(tmp)
+            return out
+        _S.paged_attention_any(out, q, k_cache, v_cache, block_tables,
+                               query_start_loc, seq_lens, float(scale),
+                               int(max_query_len))
+        return out
+    out.copy_(reference.paged_attention(
+        q, k_cache, v_cache, block_tables.cpu(), query_start_loc.cpu(),
+        seq_lens.cpu(), scale))
+    return out
+
+
+def gqa_attention_decode(q, k_cache, v_cache, block_tables, seq_lens, scale,
+                         out: torch.Tensor) -> torch.Tensor:
+    """Same attention for one new query per sequence (seq_len 0 = padding row,
+    zeros)."""
+    if q.numel() and _native_seq(q):
+        if _matrix_core_attention_fits(q, k_cache, v_cache):
+            if out.is_contiguous():
+                _C.paged_attention_decode(out, q, k_cache, v_cache, block_tables,
+                                          seq_lens, float(scale))
+            else:
+                tmp = torch.empty_like(q)
+                _C.paged_attention_decode(tmp, q, k_cache, v_cache, block_tables,
+                                          seq_lens, float(scale))
+                out.copy_(tmp)
+            return out
+        _S.paged_attention_any(out, q, k_cache, v_cache, block_tables, None,
+                               seq_lens, float(scale), 1)
+        return out
+    n = q.shape[0]
+    qsl = torch.arange(n + 1, dtype=torch.int32)
+    out.copy_(reference.paged_attention(
+        q, k_cache, v_cache, block_tables.cpu(), qsl, seq_lens.cpu(), scale))
+    return out
+
+
+def ssd_scan(xbc, dt, dt_bias, a_log, d_skip, state, seq_start_loc, seq_lens,
+             state_slots, heads: int, vdim: int, nstate: int, groups: int) -> torch.Tensor:
+    """State-space-duality recurrence over each sequence's new rows with the
+    f32 state [slots, H, N, vdim] advanced in place; returns y [T, H*vdim] f32."""
+    if xbc.numel() and _native_seq(xbc):
+        y = torch.empty((xbc.shape[0], heads * vdim), dtype=torch.float32,
+                        device=xbc.device)
+        _S.ssd_scan(y, xbc, dt, dt_bias, a_log, d_skip, state, seq_start_loc,
+                    seq_lens, state_slots, int(heads), int(vdim), int(nstate),
+                    int(groups))
+        return y
+    return reference.ssd_scan(xbc, dt, dt_bias, a_log, d_skip, state,
+                              seq_start_loc.cpu(), seq_lens.cpu(), state_slots.cpu(),
+                              heads, vdim, nstate, groups)
+
+
+def gated_group_norm(y, gate, weight, groups: int, eps: float, gate_first: bool,
+                     out_dtype: torch.dtype) -> torch.Tensor:
+    """RMS norm of y [T, C] (f32) in ``groups`` equal parts, times weight, with
+    a gate [T, C]: silu(gate) multiplied in before the norm (gate_first) or
+    sigmoid(gate) after it."""
+    if y.numel() and _native_seq(y):
+        out = torch.empty(y.shape, dtype=out_dtype, device=y.device)
+        _S.gated_group_norm(out, y, gate, weight, int(groups), float(eps),
+                            bool(gate_first))
+        return out
+    return reference.gated_group_norm(y, gate, weight, groups, eps, gate_first, out_dtype)
+
+
+def rglru_scan(u, r_pre, i_pre, r_bias, i_bias, lam, gate_c, y_branch, state,
+               seq_start_loc, seq_lens, state_slots) -> torch.Tensor:
+    """Real-gated linear recurrent unit over each sequence's new rows (f32
+    state [slots, W] advanced in place), times the other branch."""
+    if u.numel() and _native_seq(u):
+        out = torch.empty(u.shape, dtype=u.dtype, device=u.device)
+        _S.rglru_scan(out, u, r_pre, i_pre, r_bias, i_bias, lam, float(gate_c),
+                      y_branch, state, seq_start_loc, seq_lens, state_slots)
+        return out
+    return reference.rglru_scan(u, r_pre, i_pre, r_bias, i_bias, lam, gate_c,
+                                y_branch, state, seq_start_loc.cpu(), seq_lens.cpu(),
+                                state_slots.cpu())
+
+
+def mlstm_scan(q, k, v, i_pre, f_pre, i_bias, f_bias, cap, q_scale, s_state,
+               n_state, m_state, seq_start_loc, seq_lens, state_slots) -> torch.Tensor:
+    """mLSTM matrix-memory recurrence over each sequence's new rows (f32 state
+    S, n, m advanced in place); returns o [T, H*vdim] f32."""
+    if q.numel() and _native_seq(q):
+        o = torch.empty((q.shape[0], q.shape[1] * v.shape[-1]), dtype=torch.float32,
+                        device=q.device)
+        _S.mlstm_scan(o, q, k, v, i_pre, f_pre, i_bias, f_bias, float(cap),
+                      float(q_scale), s_state, n_state, m_state, seq_start_loc,
+                      seq_lens, state_slots)
+        return o
+    return reference.mlstm_scan(q, k, v, i_pre, f_pre, i_bias, f_bias, cap, q_scale,
+                                s_state, n_state, m_state, seq_start_loc.cpu(),
+                                seq_lens.cpu(), state_slots.cpu())

@@ -120,13 +120,18 @@ def paged_attention(
     num_heads = q.shape[1]
     num_kv_heads = k_cache.shape[2]
     group = num_heads // num_kv_heads
-    out = torch.empty_like(q)
+    # the value size may differ from the query/key size
+    out = torch.empty((q.shape[0], num_heads, v_cache.shape[-1]), dtype=q.dtype,
+                      device=q.device)
     qs = query_start_loc.tolist()
     lens = seq_lens.tolist()
     for i in range(len(lens)):
         s, e = qs[i], qs[i + 1]
         q_len = e - s
         seq_len = lens[i]
+        if q_len == 0 or seq_len == 0:
+            out[s:e] = 0
+            continue
         k, v = _gather_kv(k_cache, v_cache, block_tables[i], seq_len)
         qf = q[s:e].float()                       # [q, H, d]
         kf = k.float().repeat_interleave(group, dim=1)  # [S, H, d]
@@ -195,20 +200,22 @@ def softcap(logits: torch.Tensor, cap: float) -> torch.Tensor:
 
 
 def causal_conv_state(
-    h: torch.Tensor,            # [T, W]
+    h: torch.Tensor,            # [T, W] (rows may be strided)
     weight: torch.Tensor,       # [W, taps]
     state: torch.Tensor,        # [slots, taps-1, W]
     seq_start_loc: torch.Tensor,  # [S+1] rows of each sequence's new tokens
     seq_lens: torch.Tensor,       # [S] tokens of the sequence incl. the new ones
     state_slots: torch.Tensor,    # [S]
     add_input: bool,
+    bias: torch.Tensor | None = None,   # [W] f32
+    act: str | None = None,             # None | "silu"
 ) -> torch.Tensor:
     """out_t = (h_t if add_input) + sum_j w[:, j] * h_(t - taps + 1 + j) per
     sequence, inputs before the step's rows come from ``state`` (the last
     taps-1 inputs of the sequence), inputs before the sequence are zero;
     ``state`` is then advanced past the new rows."""
     taps = weight.shape[1]
-    out = torch.empty_like(h)
+    out = torch.empty(h.shape, dtype=h.dtype, device=h.device)
     loc = seq_start_loc.tolist()
     lens = seq_lens.tolist()
     slots = state_slots.tolist()
@@ -217,6 +224,9 @@ def causal_conv_state(
         a, b = loc[i], loc[i + 1]
         n = b - a
         if n == 0:
+            continue
+        if slots[i] < 0:
+            out[a:b] = 0
             continue
         start = lens[i] - n
         hist = state[slots[i]].float() if taps > 1 else h.new_zeros((0, h.shape[1]), dtype=torch.float32)
@@ -228,6 +238,10 @@ def causal_conv_state(
         acc = h[a:b].float().clone() if add_input else torch.zeros_like(ext[taps - 1:])
         for j in range(taps):
             acc = acc + wf[:, j] * ext[j:j + n]
+        if bias is not None:
+            acc = acc + bias.float()
+        if act == "silu":
+            acc = acc * torch.sigmoid(acc)
         out[a:b] = acc.to(h.dtype)
         if taps > 1:
             state[slots[i]] = ext[n:].to(state.dtype)
@@ -318,3 +332,237 @@ def latent_attention(
         p = p / den.unsqueeze(-1)
         out[s:e] = torch.einsum("hqs,sd->qhd", p, kv[:, :rank]).to(out.dtype)
     return out
+
+
+# ---------------------------------------------------------------------------
+# Layer norm of an f32 stream, per-head query/key RMS norm with a query
+# temperature, recurrent mixers with per-sequence f32 state (matrix-state
+# scans of the SSD and mLSTM kind, the gated linear recurrent unit)
+# ---------------------------------------------------------------------------
+
+
+def _layer_norm_f32(xf: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    mu = xf.mean(dim=-1, keepdim=True)
+    d = xf - mu
+    var = (d * d).mean(dim=-1, keepdim=True)
+    return d * torch.rsqrt(var + eps) * weight.float()
+
+
+def layer_norm_stream(x: torch.Tensor, weight: torch.Tensor, eps: float,
+                      out_dtype: torch.dtype) -> torch.Tensor:
+    """Bias-free layer norm of an f32 stream into the compute dtype."""
+    return _layer_norm_f32(x.float(), weight, eps).to(out_dtype)
+
+
+def stream_add_layer_norm(x: torch.Tensor, a: torch.Tensor, b: torch.Tensor | None,
+                          scale_a: float, scale_b: float, weight: torch.Tensor,
+                          layer_scale: torch.Tensor | None, eps: float) -> None:
+    """x (f32, in place) += LN(scale_a * a + scale_b * b) * weight * layer_scale."""
+    y = a.float() * scale_a
+    if b is not None:
+        y = y + b.float() * scale_b
+    y = _layer_norm_f32(y, weight, eps)
+    if layer_scale is not None:
+        y = y * layer_scale.float()
+    x.add_(y)
+
+
+def stream_add_vec(x: torch.Tensor, other: torch.Tensor | None, vec: torch.Tensor) -> None:
+    """x (f32, in place) += other + vec (vec broadcast over rows)."""
+    if other is not None:
+        x.add_(other)
+    x.add_(vec.float())
+
+
+def qk_norm_cache_write(
+    q: torch.Tensor,            # [T, H, dim]  (may be a strided view)
+    k: torch.Tensor,            # [T, G, dim]
+    v: torch.Tensor,            # [T, G, vdim]
+    q_weight: torch.Tensor,     # [dim] f32
+    k_weight: torch.Tensor,     # [dim] f32
+    eps: float,
+    positions: torch.Tensor,    # [T] int64
+    temp_coef: float,
+    temp_every: int,            # 0 = no query temperature
+    k_cache: torch.Tensor,      # [blocks, block, G, dim]
+    v_cache: torch.Tensor,      # [blocks, block, G, vdim]
+    slot_mapping: torch.Tensor,
+) -> torch.Tensor:
+    """Per-head RMS norm of queries and keys (f32 statistics, plain weight);
+    queries are then multiplied by 1 + coef * ln(floor((p + 1) / every) + 1);
+    normed keys and the values go to the paged cache.  Returns the queries
+    [T, H, dim] (contiguous)."""
+    qf = q.float()
+    qf = qf * torch.rsqrt(qf.pow(2).mean(dim=-1, keepdim=True) + eps) * q_weight.float()
+    if temp_every > 0:
+        p = positions.to(torch.float32)
+        temp = 1.0 + temp_coef * torch.log(torch.floor((p + 1.0) / temp_every) + 1.0)
+        qf = qf * temp.view(-1, 1, 1)
+    kf = k.float()
+    kf = kf * torch.rsqrt(kf.pow(2).mean(dim=-1, keepdim=True) + eps) * k_weight.float()
+    ok = slot_mapping >= 0
+    sm = slot_mapping[ok]
+    bs = k_cache.shape[1]
+    blk = torch.div(sm, bs, rounding_mode="floor")
+    k_cache[blk, sm % bs] = kf[ok].to(k_cache.dtype)
+    v_cache[blk, sm % bs] = v[ok].to(v_cache.dtype)
+    return qf.to(q.dtype).contiguous()
+
+
+def _softplus(z: torch.Tensor) -> torch.Tensor:
+    return torch.nn.functional.softplus(z, beta=1.0, threshold=30.0)
+
+
+def _seq_iter(seq_start_loc, seq_lens, state_slots):
+    loc = seq_start_loc.tolist()
+    lens = seq_lens.tolist()
+    slots = state_slots.tolist()
+    for i in range(len(lens)):
+        a, b = loc[i], loc[i + 1]
+        if b > a:
+            yield a, b, lens[i] - (b - a), slots[i]
+
+
+def ssd_scan(
+    xbc: torch.Tensor,          # [T, inner + 2*G*N] after convolution + activation
+    dt: torch.Tensor,           # [T, H] raw step sizes (may be a strided view)
+    dt_bias: torch.Tensor,      # [H] f32
+    a_log: torch.Tensor,        # [H] f32
+    d_skip: torch.Tensor,       # [H] f32
+    state: torch.Tensor,        # [slots, H, N, vdim] f32
+    seq_start_loc, seq_lens, state_slots,
+    heads: int, vdim: int, nstate: int, groups: int,
+) -> torch.Tensor:
+    """S_t = exp(-exp(A_log) * dt_t) S_(t-1) + dt_t * B_t x_t^T, y_t = S_t^T C_t
+    + D x_t per head, dt_t = softplus(dt + dt_bias); f32 throughout; a sequence
+    that starts in this step starts from S = 0 whatever its slot holds.
+    Returns y [T, H*vdim] f32."""
+    t = xbc.shape[0]
+    inner = heads * vdim
+    y = torch.zeros((t, heads, vdim), dtype=torch.float32, device=xbc.device)
+    xf = xbc.float()
+    dtf = _softplus(dt.float() + dt_bias.float())
+    decay = torch.exp(-torch.exp(a_log.float()) * dtf)          # [T, H]
+    per = heads // groups
+    for a, b, start, slot in _seq_iter(seq_start_loc, seq_lens, state_slots):
+        if slot < 0:
+            continue
+        s = state[slot].clone() if start > 0 else torch.zeros_like(state[slot])
+        for i in range(a, b):
+            x = xf[i, :inner].view(heads, vdim)
+            bm = xf[i, inner:inner + groups * nstate].view(groups, nstate)
+            cm = xf[i, inner + groups * nstate:].view(groups, nstate)
+            bm = bm.repeat_interleave(per, dim=0)               # [H, N]
+            cm = cm.repeat_interleave(per, dim=0)
+            s = decay[i].view(heads, 1, 1) * s \
+                + (dtf[i].view(heads, 1) * bm).unsqueeze(2) * x.unsqueeze(1)
+            y[i] = torch.einsum("hnv,hn->hv", s, cm) + d_skip.float().view(heads, 1) * x
+        state[slot] = s
+    return y.view(t, inner)
+
+
+def gated_group_norm(
+    y: torch.Tensor,            # [T, C] f32
+    gate: torch.Tensor,         # [T, C] compute dtype (may be a strided view)
+    weight: torch.Tensor,       # [C] f32
+    groups: int,
+    eps: float,
+    gate_first: bool,
+    out_dtype: torch.dtype,
+) -> torch.Tensor:
+    """gate_first: RMS-norm of y * silu(gate) in ``groups`` equal parts, times
+    weight.  Otherwise: RMS-norm of y in parts, times weight, times
+    sigmoid(gate)."""
+    t, c = y.shape
+    yf = y.float()
+    gf = gate.float()
+    if gate_first:
+        yf = yf * (gf * torch.sigmoid(gf))
+    yg = yf.view(t, groups, c // groups)
+    yg = yg * torch.rsqrt(yg.pow(2).mean(dim=-1, keepdim=True) + eps)
+    out = yg.reshape(t, c) * weight.float()
+    if not gate_first:
+        out = out * torch.sigmoid(gf)
+    return out.to(out_dtype)
+
+
+def rglru_scan(
+    u: torch.Tensor,            # [T, W] convolved input branch
+    r_pre: torch.Tensor,        # [T, W] recurrence-gate pre-activation (no bias)
+    i_pre: torch.Tensor,        # [T, W] input-gate pre-activation (no bias)
+    r_bias: torch.Tensor,       # [W] f32
+    i_bias: torch.Tensor,       # [W] f32
+    lam: torch.Tensor,          # [W] f32
+    gate_c: float,              # the constant in log a = -c * r * softplus(lam)
+    y_branch: torch.Tensor,     # [T, W] the other branch, multiplied in at the end
+    state: torch.Tensor,        # [slots, W] f32
+    seq_start_loc, seq_lens, state_slots,
+) -> torch.Tensor:
+    """S_t = a_t S_(t-1) + sqrt(1 - a_t^2) * i_t * u_t with a_t = exp(-c * r_t *
+    softplus(lam)); returns S_t * y_t in u's dtype."""
+    uf = u.float()
+    r = torch.sigmoid(r_pre.float() + r_bias.float())
+    g = torch.sigmoid(i_pre.float() + i_bias.float())
+    log_a = -gate_c * r * _softplus(lam.float())
+    a_ = torch.exp(log_a)
+    inp = torch.sqrt(1.0 - a_ * a_) * g * uf
+    out = torch.zeros(u.shape, dtype=torch.float32, device=u.device)
+    for a, b, start, slot in _seq_iter(seq_start_loc, seq_lens, state_slots):
+        if slot < 0:
+            continue
+        s = state[slot].clone() if start > 0 else torch.zeros_like(state[slot])
+        for i in range(a, b):
+            s = a_[i] * s + inp[i]
+            out[i] = s
+        state[slot] = s
+    return (out * y_branch.float()).to(u.dtype)
+
+
+def mlstm_scan(
+    q: torch.Tensor,            # [T, H, dim]
+    k: torch.Tensor,            # [T, H, dim]
+    v: torch.Tensor,            # [T, H, vdim]
+    i_pre: torch.Tensor,        # [T, H] input-gate pre-activation (no bias)
+    f_pre: torch.Tensor,        # [T, H] forget-gate pre-activation (no bias)
+    i_bias: torch.Tensor,       # [H] f32
+    f_bias: torch.Tensor,       # [H] f32
+    cap: float,
+    q_scale: float,
+    s_state: torch.Tensor,      # [slots, H, dim, vdim] f32
+    n_state: torch.Tensor,      # [slots, H, dim] f32
+    m_state: torch.Tensor,      # [slots, H] f32
+    seq_start_loc, seq_lens, state_slots,
+) -> torch.Tensor:
+    """Matrix memory with exponential gates held stable by a running maximum m
+    (m = 0 before the first token): i = cap * tanh((i_pre + b) / cap), f =
+    logsigmoid(cap * tanh((f_pre + b) / cap)), m_t = max(f + m, i), S_t =
+    exp(f + m - m_t) S + exp(i - m_t) k v^T, n_t likewise with k, o = S_t^T q /
+    (max(|n_t . q|, exp(-m_t)) + 1e-6).  Returns o [T, H*vdim] f32."""
+    t, heads, dim = q.shape
+    vdim = v.shape[-1]
+    qf = q.float() * q_scale
+    kf, vf = k.float(), v.float()
+    ig = cap * torch.tanh((i_pre.float() + i_bias.float()) / cap)
+    fg = torch.nn.functional.logsigmoid(
+        cap * torch.tanh((f_pre.float() + f_bias.float()) / cap))
+    o = torch.zeros((t, heads, vdim), dtype=torch.float32, device=q.device)
+    for a, b, start, slot in _seq_iter(seq_start_loc, seq_lens, state_slots):
+        if slot < 0:
+            continue
+        if start > 0:
+            s, n, m = s_state[slot].clone(), n_state[slot].clone(), m_state[slot].clone()
+        else:
+            s = torch.zeros_like(s_state[slot])
+            n = torch.zeros_like(n_state[slot])
+            m = torch.zeros_like(m_state[slot])
+        for i in range(a, b):
+            m_new = torch.maximum(fg[i] + m, ig[i])
+            fd = torch.exp(fg[i] + m - m_new)
+            idc = torch.exp(ig[i] - m_new)
+            s = fd.view(heads, 1, 1) * s + idc.view(heads, 1, 1) * kf[i].unsqueeze(2) * vf[i].unsqueeze(1)
+            n = fd.view(heads, 1) * n + idc.view(heads, 1) * kf[i]
+            m = m_new
+            den = torch.maximum((n * qf[i]).sum(dim=-1).abs(), torch.exp(-m)) + 1e-6
+            o[i] = torch.einsum("hdv,hd->hv", s, qf[i]) / den.view(heads, 1)
+        s_state[slot], n_state[slot], m_state[slot] = s, n, m
+    return o.view(t, heads * vdim)
