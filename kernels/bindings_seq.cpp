@@ -33,7 +33,10 @@ void launch_latent_kv_write(const T*, const float*, float, const long*,
 template <typename T>
 void launch_causal_conv_state(T*, const T*, const float*, T*, const int*,
                               const int*, const int*, int, int, int, int, int,
-                              hipStream_t);
+                              long, const float*, int, hipStream_t);
+// layer norms of the stream, attention of any shape, recurrences
+// (bindings_rec.cpp)
+void register_rec_ops(pybind11::module& m);
 template <typename T>
 void launch_latent_attention(T*, long, long, const T*, long, long, const T*,
                              long, long, const T*, const int*, int, const int*,
@@ -241,9 +244,16 @@ void latent_kv_write(torch::Tensor dkv, torch::Tensor norm_w, double eps,
 void causal_conv_state(torch::Tensor out, torch::Tensor h, torch::Tensor weight,
                        torch::Tensor state, torch::Tensor loc,
                        torch::Tensor seq_lens, torch::Tensor slots,
-                       bool add_input) {
-  TORCH_CHECK(h.is_cuda() && h.is_contiguous() && h.dim() == 2 &&
-              out.is_contiguous() && out.scalar_type() == h.scalar_type());
+                       bool add_input, c10::optional<torch::Tensor> bias,
+                       int64_t act) {
+  TORCH_CHECK(h.is_cuda() && h.dim() == 2 && h.stride(1) == 1 &&
+              out.is_contiguous() && out.scalar_type() == h.scalar_type() &&
+              out.numel() == h.numel());
+  if (bias.has_value()) {
+    check_f32(bias.value(), "bias");
+    TORCH_CHECK(bias.value().numel() == h.size(1));
+  }
+  TORCH_CHECK(act == 0 || act == 1, "act: 0 = none, 1 = silu");
   check_f32(weight, "weight");
   check_i32(loc, "seq_start_loc");
   check_i32(seq_lens, "seq_lens");
@@ -260,7 +270,9 @@ void causal_conv_state(torch::Tensor out, torch::Tensor h, torch::Tensor weight,
     launch_causal_conv_state<scalar_t>(
         ptr<scalar_t>(out), ptr<scalar_t>(h), ptr<float>(weight),
         ptr<scalar_t>(state), ptr<int>(loc), ptr<int>(seq_lens), ptr<int>(slots),
-        (int)h.size(0), nseq, width, taps, add_input ? 1 : 0, stream());
+        (int)h.size(0), nseq, width, taps, add_input ? 1 : 0, (long)h.stride(0),
+        bias.has_value() ? ptr<float>(bias.value()) : nullptr, (int)act,
+        stream());
   });
 }
 
@@ -376,4 +388,5 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("causal_conv_state", &causal_conv_state);
   m.def("latent_attention_prefill", &latent_attention_prefill);
   m.def("latent_attention_decode", &latent_attention_decode);
+  register_rec_ops(m);
 }

@@ -9,8 +9,10 @@ Two extensions, so that a model only needs the one it uses:
 
 ``_C``    the llama/mixtral/opt kernel set (every kernels/*.hip that is not
           listed for another extension) + bindings.cpp
-``_C_seq`` f32-residual-stream ops, short causal convolution with per-sequence
-          state, windowed latent attention with sinks + bindings_seq.cpp
+``_C_seq`` f32-residual-stream ops (RMS and layer norms), short causal
+          convolution with per-sequence state, windowed latent attention with
+          sinks, grouped-query attention of any shape, recurrences with
+          per-sequence state + bindings_seq.cpp, bindings_rec.cpp
 """
 
 from __future__ import annotations
@@ -28,7 +30,8 @@ PKG = REPO / "vllm_tgis_adapter_amd"
 ARCH = os.environ.get("PYTORCH_ROCM_ARCH", "gfx950")
 
 _SEQ_SOURCES = ["stream_ops.hip", "canon_conv.hip", "latent_attention.hip",
-                "latent_attention_mfma.hip"]
+                "latent_attention_mfma.hip", "layer_norm_stream.hip",
+                "paged_attention_any.hip", "recurrent_scan.hip"]
 
 EXTENSIONS = {
     "_C": dict(
@@ -37,7 +40,8 @@ EXTENSIONS = {
     ),
     "_C_seq": dict(
         sources=lambda: [KERNELS / n for n in _SEQ_SOURCES
-                         if (KERNELS / n).exists()] + [KERNELS / "bindings_seq.cpp"],
+                         if (KERNELS / n).exists()]
+        + [KERNELS / "bindings_seq.cpp", KERNELS / "bindings_rec.cpp"],
     ),
 }
 OUT = PKG / "_C.so"

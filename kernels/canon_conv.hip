@@ -1,6 +1,9 @@
 // Short depthwise causal convolution over time with per-sequence state.
 //
-//   out_t = [h_t +] sum_j w[:, j] * h_(t - taps + 1 + j)
+//   out_t = act([h_t +] sum_j w[:, j] * h_(t - taps + 1 + j) [+ bias])
+//
+// act is the identity or silu; the input rows may be a column slice of a wider
+// matrix (row stride in_st), output and state rows are dense.
 //
 // A step brings, for each sequence, rows [loc[s], loc[s+1]) of new inputs that
 // continue the sequence at position start = seq_len - n.  Inputs older than the
@@ -62,7 +65,9 @@ __global__ void causal_conv_kernel(T* __restrict__ out, const T* __restrict__ h,
                                    const int* __restrict__ loc,
                                    const int* __restrict__ seq_lens,
                                    const int* __restrict__ slots, int nseq,
-                                   int width, int taps, int add_input) {
+                                   int width, int taps, int add_input,
+                                   long in_st, const float* __restrict__ bias,
+                                   int act) {
   const int row = blockIdx.x;
   const int c = (blockIdx.y * blockDim.x + threadIdx.x) * CH;
   if (c >= width) return;
@@ -89,7 +94,7 @@ __global__ void causal_conv_kernel(T* __restrict__ out, const T* __restrict__ h,
     }
   }
   if (add_input) {
-    load_ch<T, CH>(h + o, acc);
+    load_ch<T, CH>(h + (long)row * in_st + c, acc);
   } else {
 #pragma unroll
     for (int k = 0; k < CH; ++k) acc[k] = 0.f;
@@ -100,7 +105,7 @@ __global__ void causal_conv_kernel(T* __restrict__ out, const T* __restrict__ h,
     if (pj < 0) continue;
     float v[CH];
     if (pj >= start)
-      load_ch<T, CH>(h + (long)(loc[s] + pj - start) * width + c, v);
+      load_ch<T, CH>(h + (long)(loc[s] + pj - start) * in_st + c, v);
     else
       load_ch<T, CH>(st + (long)(pj - (start - (taps - 1))) * width + c, v);
 #pragma unroll
@@ -108,6 +113,14 @@ __global__ void causal_conv_kernel(T* __restrict__ out, const T* __restrict__ h,
       const float wk = (TAPS > 0 && CH == 4) ? wreg[k * TAPS + j] : w[(c + k) * taps + j];
       acc[k] += wk * v[k];
     }
+  }
+  if (bias != nullptr) {
+#pragma unroll
+    for (int k = 0; k < CH; ++k) acc[k] += bias[c + k];
+  }
+  if (act == 1) {
+#pragma unroll
+    for (int k = 0; k < CH; ++k) acc[k] = acc[k] / (1.0f + expf(-acc[k]));
   }
   store_ch<T, CH>(out + o, acc);
 }
@@ -118,7 +131,7 @@ __global__ void conv_state_update_kernel(T* __restrict__ state,
                                          const int* __restrict__ loc,
                                          const int* __restrict__ seq_lens,
                                          const int* __restrict__ slots,
-                                         int width, int taps) {
+                                         int width, int taps, long in_st) {
   const int s = blockIdx.x;
   const int c = blockIdx.y * blockDim.x + threadIdx.x;
   if (c >= width) return;
@@ -133,7 +146,7 @@ __global__ void conv_state_update_kernel(T* __restrict__ state,
     const int pj = end - (taps - 1) + j;
     T v = ScalarOps<T>::from_f32(0.f);
     if (pj >= start)
-      v = h[(long)(loc[s] + pj - start) * width + c];
+      v = h[(long)(loc[s] + pj - start) * in_st + c];
     else if (pj >= 0)
       v = st[(long)(j + n) * width + c];
     st[(long)j * width + c] = v;
@@ -144,9 +157,11 @@ template <typename T>
 void launch_causal_conv_state(T* out, const T* h, const float* w, T* state,
                               const int* loc, const int* seq_lens,
                               const int* slots, int rows, int nseq, int width,
-                              int taps, int add_input, hipStream_t stream) {
+                              int taps, int add_input, long in_st,
+                              const float* bias, int act, hipStream_t stream) {
   const int block = 256;
-  const bool vec = width % 4 == 0 &&
+  const bool vec = width % 4 == 0 && in_st % 4 == 0 &&
+                   (bias == nullptr || reinterpret_cast<uintptr_t>(bias) % 16 == 0) &&
                    reinterpret_cast<uintptr_t>(h) % (4 * sizeof(T)) == 0 &&
                    reinterpret_cast<uintptr_t>(state) % (4 * sizeof(T)) == 0 &&
                    reinterpret_cast<uintptr_t>(w) % 16 == 0;
@@ -154,7 +169,8 @@ void launch_causal_conv_state(T* out, const T* h, const float* w, T* state,
     dim3 g1(rows, (width / 4 + block - 1) / block);
 #define CONV_LAUNCH(TP)                                                        \
     causal_conv_kernel<T, 4, TP><<<g1, block, 0, stream>>>(                    \
-        out, h, w, state, loc, seq_lens, slots, nseq, width, taps, add_input)
+        out, h, w, state, loc, seq_lens, slots, nseq, width, taps, add_input, \
+        in_st, bias, act)
     switch (taps) {
       case 2: CONV_LAUNCH(2); break;
       case 3: CONV_LAUNCH(3); break;
@@ -165,19 +181,22 @@ void launch_causal_conv_state(T* out, const T* h, const float* w, T* state,
   } else {
     dim3 g1(rows, (width + block - 1) / block);
     causal_conv_kernel<T, 1, 0><<<g1, block, 0, stream>>>(
-        out, h, w, state, loc, seq_lens, slots, nseq, width, taps, add_input);
+        out, h, w, state, loc, seq_lens, slots, nseq, width, taps, add_input,
+        in_st, bias, act);
   }
   if (taps > 1) {
     dim3 g2(nseq, (width + block - 1) / block);
     conv_state_update_kernel<T><<<g2, block, 0, stream>>>(
-        state, h, loc, seq_lens, slots, width, taps);
+        state, h, loc, seq_lens, slots, width, taps, in_st);
   }
 }
 
 template void launch_causal_conv_state<float>(float*, const float*, const float*,
                                               float*, const int*, const int*,
                                               const int*, int, int, int, int,
-                                              int, hipStream_t);
+                                              int, long, const float*, int,
+                                              hipStream_t);
 template void launch_causal_conv_state<__hip_bfloat16>(
     __hip_bfloat16*, const __hip_bfloat16*, const float*, __hip_bfloat16*,
-    const int*, const int*, const int*, int, int, int, int, int, hipStream_t);
+    const int*, const int*, const int*, int, int, int, int, int, long,
+    const float*, int, hipStream_t);

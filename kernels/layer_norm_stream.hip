@@ -1,0 +1,254 @@
+// Layer-norm flavoured ops around an f32 residual stream, and the row norms of
+// the recurrent mixers.
+//
+//   layer_norm_stream        out = (x - mean) / sqrt(var + eps) * w   (no bias)
+//   stream_add_layer_norm    x += LN(sa * a + sb * b) * w * ls, optionally also
+//                            next_out = LN(x) * next_w of the updated row
+//   stream_add_vec           x += other + vec (vec broadcast over rows)
+//   gated_group_norm         RMS norm of an f32 row in equal parts with a gate:
+//                            silu(gate) before the norm or sigmoid(gate) after
+//   qk_norm_cache_write      per-head RMS norm of queries and keys, query
+//                            temperature by position, keys and values stored
+//                            in the paged cache
+//
+// All are memory-bound row kernels: one workgroup per row (or per row part),
+// statistics in f32 with the variance taken as the mean of squared deviations
+// from the mean (second pass over the row, which sits in L1/L2 by then).  Each
+// thread touches the same columns in every pass, so a row that is updated in
+// place needs no barrier between the update and the pass that reads it back.
+
+#include "common.h"
+
+namespace {
+
+// every reduction of a kernel gets its own scratch: block_reduce_sum leaves
+// its result in scratch[0], which a following reduction would overwrite while
+// slower waves still read it
+DEVINLINE float reduce_sum(float x, float* scratch) { return block_reduce_sum(x, scratch); }
+
+template <typename T>
+__global__ __launch_bounds__(256) void layer_norm_stream_kernel(
+    T* __restrict__ out, const float* __restrict__ x, const float* __restrict__ w,
+    float eps, int width) {
+  __shared__ float r0[16], r1[16];
+  const long row = blockIdx.x;
+  const float* xr = x + row * width;
+  float s = 0.f;
+  for (int c = threadIdx.x; c < width; c += blockDim.x) s += xr[c];
+  const float mu = reduce_sum(s, r0) / width;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    const float d = xr[c] - mu;
+    ss += d * d;
+  }
+  const float inv = 1.0f / sqrtf(reduce_sum(ss, r1) / width + eps);
+  for (int c = threadIdx.x; c < width; c += blockDim.x)
+    out[row * width + c] = ScalarOps<T>::from_f32((xr[c] - mu) * inv * w[c]);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void stream_add_layer_norm_kernel(
+    float* __restrict__ x, const T* __restrict__ a, const T* __restrict__ b,
+    float sa, float sb, const float* __restrict__ w, const float* __restrict__ ls,
+    float eps, int width, T* __restrict__ next_out, const float* __restrict__ next_w,
+    float next_eps) {
+  __shared__ float r0[16], r1[16], r2[16], r3[16];
+  const long row = blockIdx.x;
+  float* xr = x + row * width;
+  const T* ar = a + row * width;
+  const T* br = b ? b + row * width : nullptr;
+  auto y_at = [&](int c) {
+    float y = sa * ScalarOps<T>::to_f32(ar[c]);
+    if (br) y += sb * ScalarOps<T>::to_f32(br[c]);
+    return y;
+  };
+  float s = 0.f;
+  for (int c = threadIdx.x; c < width; c += blockDim.x) s += y_at(c);
+  const float mu = reduce_sum(s, r0) / width;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    const float d = y_at(c) - mu;
+    ss += d * d;
+  }
+  const float inv = 1.0f / sqrtf(reduce_sum(ss, r1) / width + eps);
+  float s2 = 0.f;
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    float v = (y_at(c) - mu) * inv * w[c];
+    if (ls) v *= ls[c];
+    const float nx = xr[c] + v;
+    xr[c] = nx;
+    s2 += nx;
+  }
+  if (next_out == nullptr) return;
+  const float mu2 = reduce_sum(s2, r2) / width;
+  float ss2 = 0.f;
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    const float d = xr[c] - mu2;
+    ss2 += d * d;
+  }
+  const float inv2 = 1.0f / sqrtf(reduce_sum(ss2, r3) / width + next_eps);
+  for (int c = threadIdx.x; c < width; c += blockDim.x)
+    next_out[row * width + c] = ScalarOps<T>::from_f32((xr[c] - mu2) * inv2 * next_w[c]);
+}
+
+__global__ void stream_add_vec_kernel(float* __restrict__ x, const float* __restrict__ other,
+                                      const float* __restrict__ vec, int width, long n) {
+  for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < n;
+       i += (long)gridDim.x * blockDim.x) {
+    float v = x[i] + vec[i % width];
+    if (other) v += other[i];
+    x[i] = v;
+  }
+}
+
+// grid (rows, groups); y [rows, C] f32, gate rows strided
+template <typename T>
+__global__ __launch_bounds__(256) void gated_group_norm_kernel(
+    T* __restrict__ out, const float* __restrict__ y, const T* __restrict__ gate,
+    long gate_stride, const float* __restrict__ w, float eps, int cols, int gsize,
+    int gate_first) {
+  __shared__ float r0[16];
+  const long row = blockIdx.x;
+  const int c0 = blockIdx.y * gsize;
+  const float* yr = y + row * cols + c0;
+  const T* gr = gate + row * gate_stride + c0;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < gsize; c += blockDim.x) {
+    float v = yr[c];
+    if (gate_first) {
+      const float g = ScalarOps<T>::to_f32(gr[c]);
+      v *= g / (1.0f + expf(-g));
+    }
+    ss += v * v;
+  }
+  const float inv = 1.0f / sqrtf(reduce_sum(ss, r0) / gsize + eps);
+  for (int c = threadIdx.x; c < gsize; c += blockDim.x) {
+    const float g = ScalarOps<T>::to_f32(gr[c]);
+    const float sg = 1.0f / (1.0f + expf(-g));
+    float v = yr[c];
+    if (gate_first) v = v * (g * sg) * inv * w[c0 + c];
+    else v = v * inv * w[c0 + c] * sg;
+    out[row * cols + c0 + c] = ScalarOps<T>::from_f32(v);
+  }
+}
+
+// One wave per (token, unit): units 0..H-1 are query heads, H..H+G-1 key
+// heads, H+G..H+2G-1 value heads.  grid (tokens, ceil(units / 4)), 256 threads.
+template <typename T>
+__global__ __launch_bounds__(256) void qk_norm_cache_write_kernel(
+    T* __restrict__ q_out, const T* __restrict__ q, long q_st,
+    const T* __restrict__ k, long k_st, const T* __restrict__ v, long v_st,
+    const float* __restrict__ qw, const float* __restrict__ kw, float eps,
+    const long* __restrict__ positions, float temp_coef, int temp_every,
+    T* __restrict__ k_cache, T* __restrict__ v_cache,
+    const long* __restrict__ slot_mapping, int heads, int kv_heads, int dim,
+    int vdim) {
+  const long t = blockIdx.x;
+  const int lane = threadIdx.x & (WAVE_SIZE - 1);
+  const int unit = blockIdx.y * (blockDim.x / WAVE_SIZE) + threadIdx.x / WAVE_SIZE;
+  if (unit >= heads + 2 * kv_heads) return;
+  const long slot = slot_mapping[t];
+  if (unit >= heads + kv_heads) {           // value head: copy into the cache
+    if (slot < 0) return;
+    const int g = unit - heads - kv_heads;
+    const T* src = v + t * v_st + (long)g * vdim;
+    T* dst = v_cache + (slot * kv_heads + g) * vdim;
+    for (int c = lane; c < vdim; c += WAVE_SIZE) dst[c] = src[c];
+    return;
+  }
+  const bool is_q = unit < heads;
+  const int hh = is_q ? unit : unit - heads;
+  if (!is_q && slot < 0) return;
+  const T* src = is_q ? q + t * q_st + (long)hh * dim : k + t * k_st + (long)hh * dim;
+  float ss = 0.f;
+  for (int c = lane; c < dim; c += WAVE_SIZE) {
+    const float x = ScalarOps<T>::to_f32(src[c]);
+    ss += x * x;
+  }
+  ss = wave_reduce_sum(ss);
+  float f = 1.0f / sqrtf(ss / dim + eps);
+  const float* w = is_q ? qw : kw;
+  T* dst;
+  if (is_q) {
+    if (temp_every > 0) {
+      const long p = positions[t];
+      f *= 1.0f + temp_coef * logf((float)((p + 1) / temp_every) + 1.0f);
+    }
+    dst = q_out + (t * heads + hh) * dim;
+  } else {
+    dst = k_cache + (slot * kv_heads + hh) * dim;
+  }
+  for (int c = lane; c < dim; c += WAVE_SIZE)
+    dst[c] = ScalarOps<T>::from_f32(ScalarOps<T>::to_f32(src[c]) * f * w[c]);
+}
+
+inline int grid_for(long n, int block) {
+  long g = (n + block - 1) / block;
+  return (int)(g < 1 ? 1 : (g > 65535 ? 65535 : g));
+}
+
+}  // namespace
+
+template <typename T>
+void launch_layer_norm_stream(T* out, const float* x, const float* w, float eps,
+                              int rows, int width, hipStream_t s) {
+  layer_norm_stream_kernel<T><<<rows, 256, 0, s>>>(out, x, w, eps, width);
+}
+
+template <typename T>
+void launch_stream_add_layer_norm(float* x, const T* a, const T* b, float sa,
+                                  float sb, const float* w, const float* ls,
+                                  float eps, int rows, int width, T* next_out,
+                                  const float* next_w, float next_eps,
+                                  hipStream_t s) {
+  stream_add_layer_norm_kernel<T><<<rows, 256, 0, s>>>(
+      x, a, b, sa, sb, w, ls, eps, width, next_out, next_w, next_eps);
+}
+
+void launch_stream_add_vec(float* x, const float* other, const float* vec,
+                           int width, long n, hipStream_t s) {
+  stream_add_vec_kernel<<<grid_for(n, 256), 256, 0, s>>>(x, other, vec, width, n);
+}
+
+template <typename T>
+void launch_gated_group_norm(T* out, const float* y, const T* gate,
+                             long gate_stride, const float* w, float eps,
+                             int rows, int cols, int groups, int gate_first,
+                             hipStream_t s) {
+  const int gsize = cols / groups;
+  const int block = gsize <= 64 ? 64 : (gsize <= 128 ? 128 : 256);
+  dim3 grid(rows, groups);
+  gated_group_norm_kernel<T><<<grid, block, 0, s>>>(out, y, gate, gate_stride, w, eps,
+                                                   cols, gsize, gate_first);
+}
+
+template <typename T>
+void launch_qk_norm_cache_write(T* q_out, const T* q, long q_st, const T* k,
+                                long k_st, const T* v, long v_st, const float* qw,
+                                const float* kw, float eps, const long* positions,
+                                float temp_coef, int temp_every, T* k_cache,
+                                T* v_cache, const long* slot_mapping, int tokens,
+                                int heads, int kv_heads, int dim, int vdim,
+                                hipStream_t s) {
+  const int units = heads + 2 * kv_heads;
+  dim3 grid(tokens, (units + 3) / 4);
+  qk_norm_cache_write_kernel<T><<<grid, 256, 0, s>>>(
+      q_out, q, q_st, k, k_st, v, v_st, qw, kw, eps, positions, temp_coef,
+      temp_every, k_cache, v_cache, slot_mapping, heads, kv_heads, dim, vdim);
+}
+
+#define INSTANTIATE(T)                                                          \
+  template void launch_layer_norm_stream<T>(T*, const float*, const float*,     \
+                                            float, int, int, hipStream_t);      \
+  template void launch_stream_add_layer_norm<T>(                                \
+      float*, const T*, const T*, float, float, const float*, const float*,     \
+      float, int, int, T*, const float*, float, hipStream_t);                   \
+  template void launch_gated_group_norm<T>(T*, const float*, const T*, long,    \
+                                           const float*, float, int, int, int,  \
+                                           int, hipStream_t);                   \
+  template void launch_qk_norm_cache_write<T>(                                  \
+      T*, const T*, long, const T*, long, const T*, long, const float*,         \
+      const float*, float, const long*, float, int, T*, T*, const long*, int,   \
+      int, int, int, int, hipStream_t);
+INSTANTIATE(float)
+INSTANTIATE(__hip_bfloat16)

@@ -1,0 +1,361 @@
+// Recurrences with per-sequence f32 state, advanced over the rows a step
+// brings for each sequence (a prompt portion or one decoded token).
+//
+// A step brings, for sequence s, rows [loc[s], loc[s+1]) that continue it at
+// position start = seq_len[s] - n.  State lives in slot-indexed f32 tensors;
+// a sequence with start == 0 starts from zero state whatever its slot holds
+// (slots are reused without clearing), slot < 0 marks a padding row of a
+// captured decode bucket (zeros out, no state touched).
+//
+// matrix_scan<KIND>: state S [vdim, N] per (sequence, head), one column of
+// the value axis per thread group:
+//     S_t[j, :] = alpha_t * S_(t-1)[j, :] + beta_t * v_t[j] * k_t[:]
+//     y_t[j]    = S_t[j, :] . q_t
+//   KIND_SSD    alpha = exp(-exp(A_log) dt), beta = dt = softplus(raw + bias),
+//               k = B, q = C (shared by the heads of a group), v = x,
+//               y += D * x
+//   KIND_MLSTM  log gates i, f (capped), running maximum m: alpha = exp(f + m
+//               - m'), beta = exp(i - m'), a normaliser n_t = alpha n + beta k,
+//               y = S q / (max(|n . q|, exp(-m')) + 1e-6)
+// The N axis is split over NSP adjacent lanes, 16 state values per lane in
+// registers (N <= 1024); a workgroup of 256 threads owns 256 / NSP value
+// columns of one (sequence, head).  State rows are stored [vdim, N] so that a
+// wave loads and stores them as one contiguous run.  The value columns are
+// independent of each other, so there is no barrier in the token loop: per
+// token a thread does 32 FMAs and log2(NSP) shuffles for the dot product.
+//
+// rglru_scan: elementwise linear recurrence, one thread per (sequence,
+// channel), gates and decay computed in f32 on the fly.
+
+#include "common.h"
+
+namespace {
+
+constexpr int NPT = 16;   // state values per thread along N
+enum { KIND_SSD = 0, KIND_MLSTM = 1 };
+
+DEVINLINE float softplus_f(float x) { return fmaxf(x, 0.f) + log1pf(expf(-fabsf(x))); }
+DEVINLINE float logsigmoid_f(float x) { return fminf(x, 0.f) - log1pf(expf(-fabsf(x))); }
+DEVINLINE float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+// 16 consecutive values p[n0 .. n0+16) of a row of length n_total as f32,
+// zeros past the end
+template <typename T>
+DEVINLINE void load_slice(const T* __restrict__ p, int n0, int n_total, bool vec,
+                          float* dst) {
+  if (vec && n0 + NPT <= n_total) {
+    constexpr int V = Vec16<T>::kElems;
+#pragma unroll
+    for (int i = 0; i < NPT; i += V) {
+      const Vec16<T> v = load16(p + n0 + i);
+#pragma unroll
+      for (int u = 0; u < V; ++u) dst[i + u] = ScalarOps<T>::to_f32(v.data[u]);
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < NPT; ++i)
+      dst[i] = (n0 + i < n_total) ? ScalarOps<T>::to_f32(p[n0 + i]) : 0.f;
+  }
+}
+
+struct ScanArgs {
+  // rows
+  const void* q; const void* k; const void* v;
+  long q_st, k_st, v_st;             // row strides (elements)
+  const void* g0; const void* g1;    // SSD: raw dt; mLSTM: i_pre, f_pre  [T, H] strided
+  long g0_st, g1_st;
+  const float* p0; const float* p1; const float* p2;  // SSD: dt_bias, A_log, D; mLSTM: i_bias, f_bias
+  float cap, q_scale;
+  float* y; long y_st;               // [T, H*vdim] f32
+  float* s_state; float* n_state; float* m_state;
+  const int* loc; const int* seq_lens; const int* slots;
+  int heads, vdim, nk, per_group;    // nk = N (SSD) or dim (mLSTM); heads per k/q group
+  int vec_ok;
+};
+
+template <typename T, int KIND, int NSP>
+__global__ __launch_bounds__(256) void matrix_scan_kernel(ScanArgs a) {
+  constexpr int JW = 256 / NSP;            // value columns per workgroup
+  const int s = blockIdx.x / a.heads;
+  const int h = blockIdx.x % a.heads;
+  const int ns = threadIdx.x % NSP;
+  const int j = blockIdx.y * JW + threadIdx.x / NSP;
+  const int row0 = a.loc[s];
+  const int n = a.loc[s + 1] - row0;
+  if (n <= 0) return;
+  const int slot = a.slots[s];
+  const bool j_ok = j < a.vdim;
+  const int jc = j_ok ? j : a.vdim - 1;     // clamped lanes compute, never store
+  if (slot < 0) {
+    if (j_ok && ns == 0)
+      for (int r = 0; r < n; ++r) a.y[(long)(row0 + r) * a.y_st + (long)h * a.vdim + j] = 0.f;
+    return;
+  }
+  const int start = a.seq_lens[s] - n;
+  const int n0 = ns * NPT;
+  const int grp = h / a.per_group;
+  const bool vec = a.vec_ok != 0;
+
+  float S[NPT], nst[NPT];
+  float m = 0.f;
+  float* srow = a.s_state + (((long)slot * a.heads + h) * a.vdim + jc) * a.nk;
+  float* nrow = KIND == KIND_MLSTM ? a.n_state + ((long)slot * a.heads + h) * a.nk : nullptr;
+  if (start > 0) {
+    load_slice<float>(srow, n0, a.nk, vec, S);
+    if (KIND == KIND_MLSTM) {
+      load_slice<float>(nrow, n0, a.nk, vec, nst);
+      m = a.m_state[(long)slot * a.heads + h];
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < NPT; ++i) { S[i] = 0.f; nst[i] = 0.f; }
+  }
+
+  float c0 = 0.f, c1 = 0.f, c2 = 0.f;
+  if (KIND == KIND_SSD) {
+    c0 = a.p0[h];               // dt bias
+    c1 = -expf(a.p1[h]);        // -A
+    c2 = a.p2[h];               // D
+  } else {
+    c0 = a.p0[h];               // input-gate bias
+    c1 = a.p1[h];               // forget-gate bias
+  }
+  const T* qp = reinterpret_cast<const T*>(a.q) + (long)grp * a.nk;
+  const T* kp = reinterpret_cast<const T*>(a.k) + (long)grp * a.nk;
+  const T* vp = reinterpret_cast<const T*>(a.v) + (long)h * a.vdim + jc;
+  const T* g0 = reinterpret_cast<const T*>(a.g0) + h;
+  const T* g1 = KIND == KIND_MLSTM ? reinterpret_cast<const T*>(a.g1) + h : nullptr;
+
+  for (int r = 0; r < n; ++r) {
+    const long row = row0 + r;
+    float kk[NPT], qq[NPT];
+    load_slice<T>(kp + row * a.k_st, n0, a.nk, vec, kk);
+    load_slice<T>(qp + row * a.q_st, n0, a.nk, vec, qq);
+    const float vj = ScalarOps<T>::to_f32(vp[row * a.v_st]);
+    float alpha, beta;
+    if (KIND == KIND_SSD) {
+      const float dt = softplus_f(ScalarOps<T>::to_f32(g0[row * a.g0_st]) + c0);
+      alpha = expf(c1 * dt);
+      beta = dt;
+    } else {
+      const float ig = a.cap * tanhf((ScalarOps<T>::to_f32(g0[row * a.g0_st]) + c0) / a.cap);
+      const float fg = logsigmoid_f(
+          a.cap * tanhf((ScalarOps<T>::to_f32(g1[row * a.g1_st]) + c1) / a.cap));
+      const float m_new = fmaxf(fg + m, ig);
+      alpha = expf(fg + m - m_new);
+      beta = expf(ig - m_new);
+      m = m_new;
+    }
+    const float bv = beta * vj;
+    float dot = 0.f, ndot = 0.f;
+#pragma unroll
+    for (int i = 0; i < NPT; ++i) {
+      S[i] = alpha * S[i] + bv * kk[i];
+      if (KIND == KIND_MLSTM) {
+        const float qs = qq[i] * a.q_scale;
+        nst[i] = alpha * nst[i] + beta * kk[i];
+        dot += S[i] * qs;
+        ndot += nst[i] * qs;
+      } else {
+        dot += S[i] * qq[i];
+      }
+    }
+    dot = group_reduce_sum<NSP>(dot);
+    float yv;
+    if (KIND == KIND_MLSTM) {
+      ndot = group_reduce_sum<NSP>(ndot);
+      yv = dot / (fmaxf(fabsf(ndot), expf(-m)) + 1e-6f);
+    } else {
+      yv = dot + c2 * vj;
+    }
+    if (j_ok && ns == 0) a.y[row * a.y_st + (long)h * a.vdim + j] = yv;
+  }
+
+  if (j_ok) {
+    if (vec && n0 + NPT <= a.nk) {
+#pragma unroll
+      for (int i = 0; i < NPT; i += 4)
+        *reinterpret_cast<float4*>(srow + n0 + i) =
+            make_float4(S[i], S[i + 1], S[i + 2], S[i + 3]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < NPT; ++i)
+        if (n0 + i < a.nk) srow[n0 + i] = S[i];
+    }
+  }
+  // the normaliser n and the maximum m are read by every workgroup of this
+  // (sequence, head) and therefore advanced by a kernel of their own, after
+  // this one, on the same stream
+}
+
+// Advances n [slots, H, dim] and m [slots, H] of the mLSTM over the step's
+// rows: one workgroup per (sequence, head), one thread per key dim.
+template <typename T>
+__global__ __launch_bounds__(256) void mlstm_norm_state_kernel(ScanArgs a) {
+  const int s = blockIdx.x / a.heads;
+  const int h = blockIdx.x % a.heads;
+  const int row0 = a.loc[s];
+  const int n = a.loc[s + 1] - row0;
+  const int slot = a.slots[s];
+  if (n <= 0 || slot < 0) return;
+  const int start = a.seq_lens[s] - n;
+  const float c0 = a.p0[h], c1 = a.p1[h];
+  const T* kp = reinterpret_cast<const T*>(a.k) + (long)h * a.nk;
+  const T* g0 = reinterpret_cast<const T*>(a.g0) + h;
+  const T* g1 = reinterpret_cast<const T*>(a.g1) + h;
+  float* nrow = a.n_state + ((long)slot * a.heads + h) * a.nk;
+  float* mp = a.m_state + (long)slot * a.heads + h;
+  const float m0 = start > 0 ? *mp : 0.f;
+  float m = m0;
+  for (int d = threadIdx.x; d < a.nk || d == threadIdx.x; d += blockDim.x) {
+    const bool ok = d < a.nk;
+    float nv = (ok && start > 0) ? nrow[d] : 0.f;
+    m = m0;
+    for (int r = 0; r < n; ++r) {
+      const long row = row0 + r;
+      const float ig = a.cap * tanhf((ScalarOps<T>::to_f32(g0[row * a.g0_st]) + c0) / a.cap);
+      const float fg = logsigmoid_f(
+          a.cap * tanhf((ScalarOps<T>::to_f32(g1[row * a.g1_st]) + c1) / a.cap));
+      const float m_new = fmaxf(fg + m, ig);
+      const float kv = ok ? ScalarOps<T>::to_f32(kp[row * a.k_st + d]) : 0.f;
+      nv = expf(fg + m - m_new) * nv + expf(ig - m_new) * kv;
+      m = m_new;
+    }
+    if (ok) nrow[d] = nv;
+  }
+  // every thread read the old maximum before this barrier
+  __syncthreads();
+  if (threadIdx.x == 0) *mp = m;
+}
+
+template <typename T, int KIND>
+void launch_matrix_scan(const ScanArgs& a, int nseq, hipStream_t stream) {
+  const int nslices = (a.nk + NPT - 1) / NPT;
+  int nsp = 1;
+  while (nsp < nslices) nsp <<= 1;
+#define SCAN_CASE(P)                                                           \
+  case P: {                                                                    \
+    dim3 grid(nseq * a.heads, (a.vdim + 256 / P - 1) / (256 / P));             \
+    matrix_scan_kernel<T, KIND, P><<<grid, 256, 0, stream>>>(a);               \
+    break;                                                                     \
+  }
+  switch (nsp) {
+    SCAN_CASE(1) SCAN_CASE(2) SCAN_CASE(4) SCAN_CASE(8) SCAN_CASE(16)
+    SCAN_CASE(32) SCAN_CASE(64)
+    default: break;   // the binding refuses N > 1024
+  }
+#undef SCAN_CASE
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void rglru_scan_kernel(
+    T* __restrict__ out, const T* __restrict__ u, const T* __restrict__ r_pre,
+    const T* __restrict__ i_pre, const float* __restrict__ r_bias,
+    const float* __restrict__ i_bias, const float* __restrict__ lam, float gate_c,
+    const T* __restrict__ y_branch, float* __restrict__ state,
+    const int* __restrict__ loc, const int* __restrict__ seq_lens,
+    const int* __restrict__ slots, int width) {
+  const int s = blockIdx.x;
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= width) return;
+  const int row0 = loc[s];
+  const int n = loc[s + 1] - row0;
+  if (n <= 0) return;
+  const int slot = slots[s];
+  if (slot < 0) {
+    for (int r = 0; r < n; ++r) out[(long)(row0 + r) * width + c] = ScalarOps<T>::from_f32(0.f);
+    return;
+  }
+  const int start = seq_lens[s] - n;
+  float S = start > 0 ? state[(long)slot * width + c] : 0.f;
+  const float rb = r_bias[c], ib = i_bias[c];
+  const float sp = -gate_c * softplus_f(lam[c]);
+  for (int r = 0; r < n; ++r) {
+    const long o = (long)(row0 + r) * width + c;
+    const float uv = ScalarOps<T>::to_f32(u[o]);
+    const float rg = sigmoid_f(ScalarOps<T>::to_f32(r_pre[o]) + rb);
+    const float ig = sigmoid_f(ScalarOps<T>::to_f32(i_pre[o]) + ib);
+    const float av = expf(sp * rg);
+    S = av * S + sqrtf(1.0f - av * av) * ig * uv;
+    out[o] = ScalarOps<T>::from_f32(S * ScalarOps<T>::to_f32(y_branch[o]));
+  }
+  state[(long)slot * width + c] = S;
+}
+
+}  // namespace
+
+template <typename T>
+void launch_ssd_scan(float* y, const T* xbc, long xbc_st, const T* dt, long dt_st,
+                     const float* dt_bias, const float* a_log, const float* d_skip,
+                     float* state, const int* loc, const int* seq_lens,
+                     const int* slots, int nseq, int heads, int vdim, int nstate,
+                     int groups, int vec_ok, hipStream_t stream) {
+  const int inner = heads * vdim;
+  ScanArgs a{};
+  a.v = xbc;                                  a.v_st = xbc_st;
+  a.k = xbc + inner;                          a.k_st = xbc_st;
+  a.q = xbc + inner + (long)groups * nstate;  a.q_st = xbc_st;
+  a.g0 = dt; a.g0_st = dt_st;
+  a.p0 = dt_bias; a.p1 = a_log; a.p2 = d_skip;
+  a.y = y; a.y_st = inner;
+  a.s_state = state;
+  a.loc = loc; a.seq_lens = seq_lens; a.slots = slots;
+  a.heads = heads; a.vdim = vdim; a.nk = nstate; a.per_group = heads / groups;
+  a.vec_ok = vec_ok;
+  launch_matrix_scan<T, KIND_SSD>(a, nseq, stream);
+}
+
+template <typename T>
+void launch_mlstm_scan(float* o, const T* q, long q_st, const T* k, long k_st,
+                       const T* v, long v_st, const T* i_pre, long i_st,
+                       const T* f_pre, long f_st, const float* i_bias,
+                       const float* f_bias, float cap, float q_scale,
+                       float* s_state, float* n_state, float* m_state,
+                       const int* loc, const int* seq_lens, const int* slots,
+                       int nseq, int heads, int dim, int vdim, int vec_ok,
+                       hipStream_t stream) {
+  ScanArgs a{};
+  a.q = q; a.q_st = q_st; a.k = k; a.k_st = k_st; a.v = v; a.v_st = v_st;
+  a.g0 = i_pre; a.g0_st = i_st; a.g1 = f_pre; a.g1_st = f_st;
+  a.p0 = i_bias; a.p1 = f_bias;
+  a.cap = cap; a.q_scale = q_scale;
+  a.y = o; a.y_st = (long)heads * vdim;
+  a.s_state = s_state; a.n_state = n_state; a.m_state = m_state;
+  a.loc = loc; a.seq_lens = seq_lens; a.slots = slots;
+  a.heads = heads; a.vdim = vdim; a.nk = dim; a.per_group = 1;
+  a.vec_ok = vec_ok;
+  launch_matrix_scan<T, KIND_MLSTM>(a, nseq, stream);
+  const int block = dim >= 256 ? 256 : ((dim + 63) / 64) * 64;
+  mlstm_norm_state_kernel<T><<<nseq * heads, block, 0, stream>>>(a);
+}
+
+template <typename T>
+void launch_rglru_scan(T* out, const T* u, const T* r_pre, const T* i_pre,
+                       const float* r_bias, const float* i_bias, const float* lam,
+                       float gate_c, const T* y_branch, float* state,
+                       const int* loc, const int* seq_lens, const int* slots,
+                       int nseq, int width, hipStream_t stream) {
+  const int block = width >= 256 ? 256 : ((width + 63) / 64) * 64;
+  dim3 grid(nseq, (width + block - 1) / block);
+  rglru_scan_kernel<T><<<grid, block, 0, stream>>>(
+      out, u, r_pre, i_pre, r_bias, i_bias, lam, gate_c, y_branch, state, loc,
+      seq_lens, slots, width);
+}
+
+#define INSTANTIATE(T)                                                          \
+  template void launch_ssd_scan<T>(float*, const T*, long, const T*, long,      \
+                                   const float*, const float*, const float*,    \
+                                   float*, const int*, const int*, const int*,  \
+                                   int, int, int, int, int, int, hipStream_t);  \
+  template void launch_mlstm_scan<T>(                                           \
+      float*, const T*, long, const T*, long, const T*, long, const T*, long,   \
+      const T*, long, const float*, const float*, float, float, float*, float*, \
+      float*, const int*, const int*, const int*, int, int, int, int, int,      \
+      hipStream_t);                                                             \
+  template void launch_rglru_scan<T>(T*, const T*, const T*, const T*,          \
+                                     const float*, const float*, const float*,  \
+                                     float, const T*, float*, const int*,       \
+                                     const int*, const int*, int, int,          \
+                                     hipStream_t);
+INSTANTIATE(float)
+INSTANTIATE(__hip_bfloat16)

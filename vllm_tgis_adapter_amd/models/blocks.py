@@ -417,7 +417,7 @@ class SSDMixer(_Mixer):
 
     def cache_shapes(self, block_size: int) -> list:
         return [("slot", (max(self.taps - 1, 0), self.conv_ch), self.dtype),
-                ("slot", (self.heads, self.nstate, self.vdim), torch.float32)]
+                ("slot", (self.heads, self.vdim, self.nstate), torch.float32)]
 
     def mix(self, proj, positions, cache, meta: AttnMetadata) -> torch.Tensor:
         conv_state, ssm_state = cache
@@ -534,7 +534,7 @@ class MLSTMMixer(_Mixer):
         self.norm.data.copy_(t["norm"].float())
 
     def cache_shapes(self, block_size: int) -> list:
-        return [("slot", (self.heads, self.dim, self.vdim), torch.float32),
+        return [("slot", (self.heads, self.vdim, self.dim), torch.float32),
                 ("slot", (self.heads, self.dim), torch.float32),
                 ("slot", (self.heads,), torch.float32)]
 

@@ -697,11 +697,12 @@ def gqa_attention_prefill(q, k_cache, v_cache, block_tables, query_start_loc,
     sizes, value size unlike the key size) on the any-shape kernel."""
     if q.numel() and _native_seq(q):
         if _matrix_core_attention_fits(q, k_cache, v_cache):
-            tmp = torch.empty_like(q)
-            _C.paged_attention_prefill(tmp, q, k_cache, v_cache, block_tables,
+            dst = out if out.is_contiguous() else torch.empty_like(q)
+            _C.paged_attention_prefill(dst, q, k_cache, v_cache, block_tables,
                                        query_start_loc, seq_lens, float(scale),
                                        int(max_query_len))
-            out.copy_(tmp)
+            if dst is not out:
+                out.copy_(dst)
             return out
         _S.paged_attention_any(out, q, k_cache, v_cache, block_tables,
                                query_start_loc, seq_lens, float(scale),
@@ -741,7 +742,7 @@ def gqa_attention_decode(q, k_cache, v_cache, block_tables, seq_lens, scale,
 def ssd_scan(xbc, dt, dt_bias, a_log, d_skip, state, seq_start_loc, seq_lens,
              state_slots, heads: int, vdim: int, nstate: int, groups: int) -> torch.Tensor:
     """State-space-duality recurrence over each sequence's new rows with the
-    f32 state [slots, H, N, vdim] advanced in place; returns y [T, H*vdim] f32."""
+    f32 state [slots, H, vdim, N] advanced in place; returns y [T, H*vdim] f32."""
     if xbc.numel() and _native_seq(xbc):
         y = torch.empty((xbc.shape[0], heads * vdim), dtype=torch.float32,
                         device=xbc.device)

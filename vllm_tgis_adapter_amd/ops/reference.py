@@ -429,7 +429,7 @@ def ssd_scan(
     dt_bias: torch.Tensor,      # [H] f32
     a_log: torch.Tensor,        # [H] f32
     d_skip: torch.Tensor,       # [H] f32
-    state: torch.Tensor,        # [slots, H, N, vdim] f32
+    state: torch.Tensor,        # [slots, H, vdim, N] f32
     seq_start_loc, seq_lens, state_slots,
     heads: int, vdim: int, nstate: int, groups: int,
 ) -> torch.Tensor:
@@ -455,8 +455,8 @@ def ssd_scan(
             bm = bm.repeat_interleave(per, dim=0)               # [H, N]
             cm = cm.repeat_interleave(per, dim=0)
             s = decay[i].view(heads, 1, 1) * s \
-                + (dtf[i].view(heads, 1) * bm).unsqueeze(2) * x.unsqueeze(1)
-            y[i] = torch.einsum("hnv,hn->hv", s, cm) + d_skip.float().view(heads, 1) * x
+                + x.unsqueeze(2) * (dtf[i].view(heads, 1) * bm).unsqueeze(1)
+            y[i] = torch.einsum("hvn,hn->hv", s, cm) + d_skip.float().view(heads, 1) * x
         state[slot] = s
     return y.view(t, inner)
 
@@ -528,7 +528,7 @@ def mlstm_scan(
     f_bias: torch.Tensor,       # [H] f32
     cap: float,
     q_scale: float,
-    s_state: torch.Tensor,      # [slots, H, dim, vdim] f32
+    s_state: torch.Tensor,      # [slots, H, vdim, dim] f32
     n_state: torch.Tensor,      # [slots, H, dim] f32
     m_state: torch.Tensor,      # [slots, H] f32
     seq_start_loc, seq_lens, state_slots,
@@ -559,10 +559,10 @@ def mlstm_scan(
             m_new = torch.maximum(fg[i] + m, ig[i])
             fd = torch.exp(fg[i] + m - m_new)
             idc = torch.exp(ig[i] - m_new)
-            s = fd.view(heads, 1, 1) * s + idc.view(heads, 1, 1) * kf[i].unsqueeze(2) * vf[i].unsqueeze(1)
+            s = fd.view(heads, 1, 1) * s + idc.view(heads, 1, 1) * vf[i].unsqueeze(2) * kf[i].unsqueeze(1)
             n = fd.view(heads, 1) * n + idc.view(heads, 1) * kf[i]
             m = m_new
             den = torch.maximum((n * qf[i]).sum(dim=-1).abs(), torch.exp(-m)) + 1e-6
-            o[i] = torch.einsum("hdv,hd->hv", s, qf[i]) / den.view(heads, 1)
+            o[i] = torch.einsum("hvd,hd->hv", s, qf[i]) / den.view(heads, 1)
         s_state[slot], n_state[slot], m_state[slot] = s, n, m
     return o.view(t, heads * vdim)
