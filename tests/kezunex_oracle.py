@@ -236,3 +236,133 @@ def forward(cfg, weights, tokens, return_layers=False):
     if return_layers:
         return logits, torch.stack(streams)
     return logits
+
+
+# ---------------------------------------------------------------------------
+# small configurations and random weights for the tests
+# ---------------------------------------------------------------------------
+
+def attn_spec(heads=4, kv_heads=2, dim=8, vdim=6, scale=0.3, coef=0.4, every=5):
+    m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale}
+    if every:
+        m["q_temp"] = {"coef": coef, "every": every}
+    return m
+
+
+def ssd_spec(heads=4, vdim=6, state=5, groups=2, conv=3, norm_groups=2):
+    return {"heads": heads, "vdim": vdim, "state": state, "groups": groups, "conv": conv,
+            "norm_groups": norm_groups}
+
+
+def layer(kind, ff=0, **kw):
+    if kind == "parallel":
+        mixer = {"left": kw.get("left") or attn_spec(), "right": kw.get("right") or ssd_spec(),
+                 "left_scale": kw.get("left_scale", 0.7), "right_scale": kw.get("right_scale", 0.4)}
+    elif kind == "rglru":
+        mixer = {"width": kw.get("width", 24), "blocks": kw.get("blocks", 3),
+                 "conv": kw.get("conv", 4)}
+    elif kind == "mlstm":
+        mixer = {"heads": kw.get("heads", 3), "dim": kw.get("dim", 4), "vdim": kw.get("vdim", 6),
+                 "gate_cap": kw.get("gate_cap", 9.0)}
+    else:
+        raise ValueError(kind)
+    return {"type": kind, "mixer": mixer, "mlp": {"kind": "dense", "ff": ff} if ff else None}
+
+
+def make_config(*, vocab=101, width=40, layers=None, loop=(1, 3, 2), eps=1e-5,
+                embed_scale=2.0) -> dict:
+    if layers is None:
+        layers = [layer("rglru"), layer("parallel", ff=48), layer("mlstm"),
+                  layer("parallel", ff=0, left=attn_spec(3, 3, 6, 10, 0.25, 0.3, 3),
+                        right=ssd_spec(2, 8, 7, 1, 2, 1))]
+    cfg = {"architecture": "Kezunex", "vocab": vocab, "width": width, "layers": layers,
+           "norm": {"eps": eps}, "embedding": {"scale": embed_scale}}
+    if loop:
+        cfg["loop"] = {"start": loop[0], "stop": loop[1], "times": loop[2]}
+    return cfg
+
+
+def make_weights(cfg: dict, seed: int = 0) -> dict:
+    """Random bf16 weights (their values are exact in f32 and f64)."""
+    g = torch.Generator().manual_seed(seed)
+    width, vocab = cfg["width"], cfg["vocab"]
+
+    def r(*shape, std=1.0, mean=0.0):
+        return (torch.randn(*shape, generator=g) * std + mean).to(torch.bfloat16)
+
+    w = {"embed": r(vocab, width, std=0.7), "final.norm": r(width, std=0.2, mean=1.0)}
+    if cfg.get("loop"):
+        w["loop.step"] = r(cfg["loop"]["times"], width, std=0.5)
+    for i, e in enumerate(cfg["layers"]):
+        p = f"l{i}."
+        for nm in ("norm1", "norm1b"):
+            w[p + nm] = r(width, std=0.2, mean=1.0)
+        w[p + "ls1"] = r(width, std=0.3, mean=0.6)
+        m = e["mixer"]
+        q = p + "mix."
+        fan = width ** -0.5
+        if e["type"] == "parallel":
+            a, s = m["left"], m["right"]
+            w[q + "left.q"] = r(a["heads"] * a["dim"], width, std=fan)
+            w[q + "left.k"] = r(a["kv_heads"] * a["dim"], width, std=fan)
+            w[q + "left.v"] = r(a["kv_heads"] * a["vdim"], width, std=fan)
+            w[q + "left.q.norm"] = r(a["dim"], std=0.3, mean=1.0)
+            w[q + "left.k.norm"] = r(a["dim"], std=0.3, mean=1.0)
+            w[q + "left.o"] = r(width, a["heads"] * a["vdim"], std=(a["heads"] * a["vdim"]) ** -0.5)
+            inner = s["heads"] * s["vdim"]
+            ch = inner + 2 * s["groups"] * s["state"]
+            w[q + "right.in"] = r(inner + ch + s["heads"], width, std=fan)
+            w[q + "right.conv"] = r(ch, s["conv"], std=0.5)
+            w[q + "right.conv.b"] = r(ch, std=0.2)
+            w[q + "right.dt_bias"] = r(s["heads"], std=1.0, mean=-1.0)
+            w[q + "right.A_log"] = r(s["heads"], std=0.7)
+            w[q + "right.D"] = r(s["heads"], std=0.5, mean=1.0)
+            w[q + "right.norm"] = r(inner, std=0.2, mean=1.0)
+            w[q + "right.o"] = r(width, inner, std=inner ** -0.5)
+        elif e["type"] == "rglru":
+            rw, nb = m["width"], m["blocks"]
+            bw = rw // nb
+            for nm in ("y", "x"):
+                w[q + nm] = r(rw, width, std=fan)
+                w[q + nm + ".b"] = r(rw, std=0.2)
+            w[q + "conv"] = r(rw, m["conv"], std=0.5)
+            w[q + "conv.b"] = r(rw, std=0.2)
+            for nm in ("ra", "ri"):
+                w[q + nm] = r(nb, bw, bw, std=bw ** -0.5)
+                w[q + nm + ".b"] = r(nb, bw, std=0.5)
+            w[q + "lam"] = r(rw, std=1.0, mean=-2.0)
+            w[q + "o"] = r(width, rw, std=rw ** -0.5)
+        else:
+            nh, d, dv = m["heads"], m["dim"], m["vdim"]
+            w[q + "q"] = r(nh * d, width, std=fan)
+            w[q + "k"] = r(nh * d, width, std=fan)
+            w[q + "v"] = r(nh * dv, width, std=fan)
+            w[q + "g"] = r(nh * dv, width, std=fan)
+            w[q + "i"] = r(nh, width, std=fan * 2)
+            w[q + "i.b"] = r(nh, std=1.0)
+            w[q + "f"] = r(nh, width, std=fan * 2)
+            w[q + "f.b"] = r(nh, std=1.0, mean=2.0)
+            w[q + "norm"] = r(nh * dv, std=0.2, mean=1.0)
+            w[q + "o"] = r(width, nh * dv, std=(nh * dv) ** -0.5)
+        if e.get("mlp"):
+            ff = e["mlp"]["ff"]
+            for nm in ("norm2", "norm2b"):
+                w[p + nm] = r(width, std=0.2, mean=1.0)
+            w[p + "ls2"] = r(width, std=0.3, mean=0.6)
+            w[p + "mlp.gate"] = r(ff, width, std=fan)
+            w[p + "mlp.up"] = r(ff, width, std=fan)
+            w[p + "mlp.down"] = r(width, ff, std=ff ** -0.5)
+    return w
+
+
+def save_model(path, cfg: dict, w: dict) -> str:
+    import json
+    import os
+
+    from safetensors.torch import save_file
+
+    os.makedirs(path, exist_ok=True)
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    save_file({k: v.contiguous() for k, v in w.items()}, os.path.join(path, "model.safetensors"))
+    return str(path)
