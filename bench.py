@@ -45,7 +45,7 @@ def parse_args():
     p.add_argument("--arch-sizes", type=str, default="s,m",
                    help="arch mode: comma list of sizes (s, m)")
     p.add_argument("--arch-models", type=str, default="dolodra,llama",
-                   help="arch mode: which of the two models to run")
+                   help="arch mode: which models to run (dolodra, kezunex, llama)")
     p.add_argument("--model", type=str, default="llama-3-8b")
     p.add_argument("--batch", type=int, default=512)
     p.add_argument("--prompt-len", type=int, default=512)
@@ -518,6 +518,50 @@ def _arch_model_configs(sz: dict, dtype: str):
     return dolo, llama
 
 
+# Kezunex at the same widths: eight layer runs (a looped pair of layers, then
+# four more), attention 128-wide heads like the llama beside it, SSD / mLSTM /
+# RG-LRU sizes in the proportions their papers use (inner size = width, state
+# 128; matrix-memory heads of dim x 2 dim; recurrent width = width).
+KEZUNEX_SIZES = {
+    "s": dict(attn=(16, 4, 128, 128), ssd=(32, 64, 128, 1), mlstm=(8, 128, 256),
+              rglru=(2048, 16), ff=5632),
+    "m": dict(attn=(32, 8, 128, 128), ssd=(64, 64, 128, 1), mlstm=(8, 256, 512),
+              rglru=(4096, 16), ff=14336),
+    "t": dict(attn=(4, 2, 16, 16), ssd=(4, 16, 16, 1), mlstm=(2, 16, 32),
+              rglru=(64, 4), ff=128),
+}
+
+
+def _kezunex_model_config(name: str, sz: dict, dtype: str):
+    from vllm_tgis_adapter_amd.engine.config import _DTYPES
+    from vllm_tgis_adapter_amd.models.kezunex import model_config_from_json
+
+    kz = KEZUNEX_SIZES[name]
+    h, g, d, dv = kz["attn"]
+    sh, sv, sn, sg = kz["ssd"]
+    mh, md, mv = kz["mlstm"]
+    rw, rb = kz["rglru"]
+    ff = {"kind": "dense", "ff": kz["ff"]}
+    par = {"type": "parallel", "mlp": ff, "mixer": {
+        "left": {"heads": h, "kv_heads": g, "dim": d, "vdim": dv, "scale": d ** -0.5,
+                 "q_temp": {"coef": 0.1, "every": 256}},
+        "right": {"heads": sh, "vdim": sv, "state": sn, "groups": sg, "conv": 4,
+                  "norm_groups": 1},
+        "left_scale": 0.5, "right_scale": 0.5}}
+    mls = {"type": "mlstm", "mlp": None,
+           "mixer": {"heads": mh, "dim": md, "vdim": mv, "gate_cap": 15.0}}
+    rec = {"type": "rglru", "mlp": None, "mixer": {"width": rw, "blocks": rb, "conv": 4}}
+    n = sz["layers"]
+    # looped [mlstm, parallel] x 2, then rglru / parallel alternating
+    layers = [mls, par] + [rec if i % 2 == 0 else par for i in range(max(n - 4, 0))]
+    hf = {"architecture": "Kezunex", "vocab": sz["vocab"], "width": sz["width"],
+          "layers": layers, "loop": {"start": 0, "stop": 2, "times": 2},
+          "norm": {"eps": 1e-5}, "embedding": {"scale": 1.0}}
+    mc = model_config_from_json("kezunex-synthetic", hf)
+    mc.dtype = _DTYPES[dtype]
+    return mc
+
+
 def _arch_measure(mc, args, device: str, batch: int, prompt_len: int, steps: int,
                   warmup: int) -> dict:
     from vllm_tgis_adapter_amd.engine import EngineConfig, LLMEngine, SamplingParams
@@ -578,9 +622,12 @@ def run_arch(args, device: str) -> None:
         plen = args.prompt_len if device == "cuda" else 32
         steps = args.steps if device == "cuda" else 4
         warm = args.warmup if device == "cuda" else 1
-        for label, mc in (("dolodra", dolo), ("llama", llama)):
+        models = [("dolodra", dolo), ("kezunex", None), ("llama", llama)]
+        for label, mc in models:
             if label not in args.arch_models.split(","):
                 continue
+            if label == "kezunex":
+                mc = _kezunex_model_config(name, sz, args.dtype)
             r = _arch_measure(mc, args, device, batch, plen, steps, warm)
             r.update(size=name, model=label, batch=batch, prompt_len=plen)
             out.append(r)

@@ -11,6 +11,10 @@
 //                            temperature by position, keys and values stored
 //                            in the paged cache
 //
+// The two stream norms keep the row in registers when the width is a multiple
+// of 4 and at most 256 * 4 * 8 (16-byte accesses, every input read once); other
+// widths take the any-width kernels, which re-read the row from L1/L2.
+//
 // All are memory-bound row kernels: one workgroup per row (or per row part),
 // statistics in f32 with the variance taken as the mean of squared deviations
 // from the mean (second pass over the row, which sits in L1/L2 by then).  Each
@@ -89,6 +93,128 @@ __global__ __launch_bounds__(256) void stream_add_layer_norm_kernel(
   const float inv2 = 1.0f / sqrtf(reduce_sum(ss2, r3) / width + next_eps);
   for (int c = threadIdx.x; c < width; c += blockDim.x)
     next_out[row * width + c] = ScalarOps<T>::from_f32((xr[c] - mu2) * inv2 * next_w[c]);
+}
+
+// ---- register-cached variants: width % 4 == 0, width <= 1024 * NCH ---------
+
+template <typename T> DEVINLINE float4 ld4(const T* p);
+template <> DEVINLINE float4 ld4<float>(const float* p) {
+  return *reinterpret_cast<const float4*>(p);
+}
+template <> DEVINLINE float4 ld4<__hip_bfloat16>(const __hip_bfloat16* p) {
+  const uint2 t = *reinterpret_cast<const uint2*>(p);
+  return make_float4(__uint_as_float(t.x << 16), __uint_as_float(t.x & 0xffff0000u),
+                     __uint_as_float(t.y << 16), __uint_as_float(t.y & 0xffff0000u));
+}
+template <typename T> DEVINLINE void st4(T* p, float4 v);
+template <> DEVINLINE void st4<float>(float* p, float4 v) {
+  *reinterpret_cast<float4*>(p) = v;
+}
+template <> DEVINLINE void st4<__hip_bfloat16>(__hip_bfloat16* p, float4 v) {
+  union { __hip_bfloat16 h[4]; uint2 u; } o;
+  o.h[0] = __float2bfloat16(v.x); o.h[1] = __float2bfloat16(v.y);
+  o.h[2] = __float2bfloat16(v.z); o.h[3] = __float2bfloat16(v.w);
+  *reinterpret_cast<uint2*>(p) = o.u;
+}
+
+// mean and 1/sqrt(var + eps) of the row held in v[NCH] (chunks past the width
+// are zero and masked out of the deviations)
+template <int NCH>
+DEVINLINE void row_stats(const float4* v, int width, float eps, float* r_a, float* r_b,
+                         float& mu, float& inv) {
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) s += (v[i].x + v[i].y) + (v[i].z + v[i].w);
+  mu = reduce_sum(s, r_a) / width;
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    if ((int)(threadIdx.x * 4 + i * 1024) < width) {
+      const float a = v[i].x - mu, b = v[i].y - mu, c = v[i].z - mu, d = v[i].w - mu;
+      ss += (a * a + b * b) + (c * c + d * d);
+    }
+  }
+  inv = 1.0f / sqrtf(reduce_sum(ss, r_b) / width + eps);
+}
+
+template <typename T, int NCH>
+__global__ __launch_bounds__(256) void layer_norm_stream_reg_kernel(
+    T* __restrict__ out, const float* __restrict__ x, const float* __restrict__ w,
+    float eps, int width) {
+  __shared__ float r0[16], r1[16];
+  const long row = blockIdx.x;
+  float4 v[NCH];
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    const int c = threadIdx.x * 4 + i * 1024;
+    v[i] = c < width ? ld4<float>(x + row * width + c) : make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+  float mu, inv;
+  row_stats<NCH>(v, width, eps, r0, r1, mu, inv);
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    const int c = threadIdx.x * 4 + i * 1024;
+    if (c < width) {
+      const float4 ww = ld4<float>(w + c);
+      st4<T>(out + row * width + c,
+             make_float4((v[i].x - mu) * inv * ww.x, (v[i].y - mu) * inv * ww.y,
+                         (v[i].z - mu) * inv * ww.z, (v[i].w - mu) * inv * ww.w));
+    }
+  }
+}
+
+template <typename T, int NCH>
+__global__ __launch_bounds__(256) void stream_add_layer_norm_reg_kernel(
+    float* __restrict__ x, const T* __restrict__ a, const T* __restrict__ b,
+    float sa, float sb, const float* __restrict__ w, const float* __restrict__ ls,
+    float eps, int width, T* __restrict__ next_out, const float* __restrict__ next_w,
+    float next_eps) {
+  __shared__ float r0[16], r1[16], r2[16], r3[16];
+  const long row = blockIdx.x;
+  float4 v[NCH];
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    const int c = threadIdx.x * 4 + i * 1024;
+    v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (c < width) {
+      const float4 t = ld4<T>(a + row * width + c);
+      v[i] = make_float4(sa * t.x, sa * t.y, sa * t.z, sa * t.w);
+      if (b != nullptr) {
+        const float4 u = ld4<T>(b + row * width + c);
+        v[i].x += sb * u.x; v[i].y += sb * u.y; v[i].z += sb * u.z; v[i].w += sb * u.w;
+      }
+    }
+  }
+  float mu, inv;
+  row_stats<NCH>(v, width, eps, r0, r1, mu, inv);
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    const int c = threadIdx.x * 4 + i * 1024;
+    if (c < width) {
+      float4 g = ld4<float>(w + c);
+      if (ls != nullptr) {
+        const float4 l = ld4<float>(ls + c);
+        g.x *= l.x; g.y *= l.y; g.z *= l.z; g.w *= l.w;
+      }
+      const float4 xo = ld4<float>(x + row * width + c);
+      v[i] = make_float4(xo.x + (v[i].x - mu) * inv * g.x, xo.y + (v[i].y - mu) * inv * g.y,
+                         xo.z + (v[i].z - mu) * inv * g.z, xo.w + (v[i].w - mu) * inv * g.w);
+      st4<float>(x + row * width + c, v[i]);
+    }
+  }
+  if (next_out == nullptr) return;
+  float mu2, inv2;
+  row_stats<NCH>(v, width, next_eps, r2, r3, mu2, inv2);
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    const int c = threadIdx.x * 4 + i * 1024;
+    if (c < width) {
+      const float4 ww = ld4<float>(next_w + c);
+      st4<T>(next_out + row * width + c,
+             make_float4((v[i].x - mu2) * inv2 * ww.x, (v[i].y - mu2) * inv2 * ww.y,
+                         (v[i].z - mu2) * inv2 * ww.z, (v[i].w - mu2) * inv2 * ww.w));
+    }
+  }
 }
 
 __global__ void stream_add_vec_kernel(float* __restrict__ x, const float* __restrict__ other,
@@ -182,6 +308,11 @@ __global__ __launch_bounds__(256) void qk_norm_cache_write_kernel(
     dst[c] = ScalarOps<T>::from_f32(ScalarOps<T>::to_f32(src[c]) * f * w[c]);
 }
 
+template <typename P>
+inline bool al16(const P* p) {   // 8 bytes are enough for 4 bf16, 16 for 4 f32
+  return p == nullptr || reinterpret_cast<uintptr_t>(p) % 16 == 0;
+}
+
 inline int grid_for(long n, int block) {
   long g = (n + block - 1) / block;
   return (int)(g < 1 ? 1 : (g > 65535 ? 65535 : g));
@@ -192,6 +323,14 @@ inline int grid_for(long n, int block) {
 template <typename T>
 void launch_layer_norm_stream(T* out, const float* x, const float* w, float eps,
                               int rows, int width, hipStream_t s) {
+  const int nch = (width + 1023) / 1024;
+  if (width % 4 == 0 && nch <= 8 && al16(out) && al16(x) && al16(w)) {
+    if (nch <= 1) layer_norm_stream_reg_kernel<T, 1><<<rows, 256, 0, s>>>(out, x, w, eps, width);
+    else if (nch <= 2) layer_norm_stream_reg_kernel<T, 2><<<rows, 256, 0, s>>>(out, x, w, eps, width);
+    else if (nch <= 4) layer_norm_stream_reg_kernel<T, 4><<<rows, 256, 0, s>>>(out, x, w, eps, width);
+    else layer_norm_stream_reg_kernel<T, 8><<<rows, 256, 0, s>>>(out, x, w, eps, width);
+    return;
+  }
   layer_norm_stream_kernel<T><<<rows, 256, 0, s>>>(out, x, w, eps, width);
 }
 
@@ -201,6 +340,19 @@ void launch_stream_add_layer_norm(float* x, const T* a, const T* b, float sa,
                                   float eps, int rows, int width, T* next_out,
                                   const float* next_w, float next_eps,
                                   hipStream_t s) {
+  const int nch = (width + 1023) / 1024;
+  if (width % 4 == 0 && nch <= 8 && al16(x) && al16(a) && al16(b) && al16(w) &&
+      al16(ls) && al16(next_out) && al16(next_w)) {
+#define SALN(N)                                                                \
+    stream_add_layer_norm_reg_kernel<T, N><<<rows, 256, 0, s>>>(               \
+        x, a, b, sa, sb, w, ls, eps, width, next_out, next_w, next_eps)
+    if (nch <= 1) SALN(1);
+    else if (nch <= 2) SALN(2);
+    else if (nch <= 4) SALN(4);
+    else SALN(8);
+#undef SALN
+    return;
+  }
   stream_add_layer_norm_kernel<T><<<rows, 256, 0, s>>>(
       x, a, b, sa, sb, w, ls, eps, width, next_out, next_w, next_eps);
 }

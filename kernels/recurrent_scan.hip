@@ -19,7 +19,8 @@
 //               y = S q / (max(|n . q|, exp(-m')) + 1e-6)
 // The N axis is split over NSP adjacent lanes, 16 state values per lane in
 // registers (N <= 1024); a workgroup of 256 threads owns 256 / NSP value
-// columns of one (sequence, head).  State rows are stored [vdim, N] so that a
+// columns of one (sequence, head), or four times as many with four columns
+// per thread (the key / query slices a thread loads then serve four columns).  State rows are stored [vdim, N] so that a
 // wave loads and stores them as one contiguous run.  The value columns are
 // independent of each other, so there is no barrier in the token loop: per
 // token a thread does 32 FMAs and log2(NSP) shuffles for the dot product.
@@ -73,22 +74,24 @@ struct ScanArgs {
   int vec_ok;
 };
 
-template <typename T, int KIND, int NSP>
+template <typename T, int KIND, int NSP, int VPT>
 __global__ __launch_bounds__(256) void matrix_scan_kernel(ScanArgs a) {
-  constexpr int JW = 256 / NSP;            // value columns per workgroup
+  constexpr int JW = 256 / NSP;            // thread groups per workgroup
   const int s = blockIdx.x / a.heads;
   const int h = blockIdx.x % a.heads;
   const int ns = threadIdx.x % NSP;
-  const int j = blockIdx.y * JW + threadIdx.x / NSP;
+  const int jbase = (blockIdx.y * JW + threadIdx.x / NSP) * VPT;   // first value column
   const int row0 = a.loc[s];
   const int n = a.loc[s + 1] - row0;
   if (n <= 0) return;
   const int slot = a.slots[s];
-  const bool j_ok = j < a.vdim;
-  const int jc = j_ok ? j : a.vdim - 1;     // clamped lanes compute, never store
   if (slot < 0) {
-    if (j_ok && ns == 0)
-      for (int r = 0; r < n; ++r) a.y[(long)(row0 + r) * a.y_st + (long)h * a.vdim + j] = 0.f;
+    if (ns == 0)
+      for (int r = 0; r < n; ++r)
+#pragma unroll
+        for (int c = 0; c < VPT; ++c)
+          if (jbase + c < a.vdim)
+            a.y[(long)(row0 + r) * a.y_st + (long)h * a.vdim + jbase + c] = 0.f;
     return;
   }
   const int start = a.seq_lens[s] - n;
@@ -96,19 +99,29 @@ __global__ __launch_bounds__(256) void matrix_scan_kernel(ScanArgs a) {
   const int grp = h / a.per_group;
   const bool vec = a.vec_ok != 0;
 
-  float S[NPT], nst[NPT];
+  // columns past vdim are clamped: they compute and never store
+  int jc[VPT];
+#pragma unroll
+  for (int c = 0; c < VPT; ++c) jc[c] = min(jbase + c, a.vdim - 1);
+
+  float S[VPT][NPT], nst[NPT];
   float m = 0.f;
-  float* srow = a.s_state + (((long)slot * a.heads + h) * a.vdim + jc) * a.nk;
-  float* nrow = KIND == KIND_MLSTM ? a.n_state + ((long)slot * a.heads + h) * a.nk : nullptr;
+  float* sbase = a.s_state + ((long)slot * a.heads + h) * a.vdim * a.nk;
+  const float* nrow = KIND == KIND_MLSTM ? a.n_state + ((long)slot * a.heads + h) * a.nk : nullptr;
   if (start > 0) {
-    load_slice<float>(srow, n0, a.nk, vec, S);
+#pragma unroll
+    for (int c = 0; c < VPT; ++c) load_slice<float>(sbase + (long)jc[c] * a.nk, n0, a.nk, vec, S[c]);
     if (KIND == KIND_MLSTM) {
       load_slice<float>(nrow, n0, a.nk, vec, nst);
       m = a.m_state[(long)slot * a.heads + h];
     }
   } else {
 #pragma unroll
-    for (int i = 0; i < NPT; ++i) { S[i] = 0.f; nst[i] = 0.f; }
+    for (int i = 0; i < NPT; ++i) {
+      nst[i] = 0.f;
+#pragma unroll
+      for (int c = 0; c < VPT; ++c) S[c][i] = 0.f;
+    }
   }
 
   float c0 = 0.f, c1 = 0.f, c2 = 0.f;
@@ -122,16 +135,17 @@ __global__ __launch_bounds__(256) void matrix_scan_kernel(ScanArgs a) {
   }
   const T* qp = reinterpret_cast<const T*>(a.q) + (long)grp * a.nk;
   const T* kp = reinterpret_cast<const T*>(a.k) + (long)grp * a.nk;
-  const T* vp = reinterpret_cast<const T*>(a.v) + (long)h * a.vdim + jc;
+  const T* vp = reinterpret_cast<const T*>(a.v) + (long)h * a.vdim;
   const T* g0 = reinterpret_cast<const T*>(a.g0) + h;
   const T* g1 = KIND == KIND_MLSTM ? reinterpret_cast<const T*>(a.g1) + h : nullptr;
 
   for (int r = 0; r < n; ++r) {
     const long row = row0 + r;
-    float kk[NPT], qq[NPT];
+    float kk[NPT], qq[NPT], vj[VPT];
     load_slice<T>(kp + row * a.k_st, n0, a.nk, vec, kk);
     load_slice<T>(qp + row * a.q_st, n0, a.nk, vec, qq);
-    const float vj = ScalarOps<T>::to_f32(vp[row * a.v_st]);
+#pragma unroll
+    for (int c = 0; c < VPT; ++c) vj[c] = ScalarOps<T>::to_f32(vp[row * a.v_st + jc[c]]);
     float alpha, beta;
     if (KIND == KIND_SSD) {
       const float dt = softplus_f(ScalarOps<T>::to_f32(g0[row * a.g0_st]) + c0);
@@ -146,41 +160,50 @@ __global__ __launch_bounds__(256) void matrix_scan_kernel(ScanArgs a) {
       beta = expf(ig - m_new);
       m = m_new;
     }
-    const float bv = beta * vj;
-    float dot = 0.f, ndot = 0.f;
+    float dot[VPT], ndot = 0.f;
+#pragma unroll
+    for (int c = 0; c < VPT; ++c) dot[c] = 0.f;
 #pragma unroll
     for (int i = 0; i < NPT; ++i) {
-      S[i] = alpha * S[i] + bv * kk[i];
+      const float bk = beta * kk[i];
+      const float qs = KIND == KIND_MLSTM ? qq[i] * a.q_scale : qq[i];
       if (KIND == KIND_MLSTM) {
-        const float qs = qq[i] * a.q_scale;
-        nst[i] = alpha * nst[i] + beta * kk[i];
-        dot += S[i] * qs;
+        nst[i] = alpha * nst[i] + bk;
         ndot += nst[i] * qs;
-      } else {
-        dot += S[i] * qq[i];
+      }
+#pragma unroll
+      for (int c = 0; c < VPT; ++c) {
+        S[c][i] = alpha * S[c][i] + bk * vj[c];
+        dot[c] += S[c][i] * qs;
       }
     }
-    dot = group_reduce_sum<NSP>(dot);
-    float yv;
+    float den = 1.f;
     if (KIND == KIND_MLSTM) {
       ndot = group_reduce_sum<NSP>(ndot);
-      yv = dot / (fmaxf(fabsf(ndot), expf(-m)) + 1e-6f);
-    } else {
-      yv = dot + c2 * vj;
+      den = 1.0f / (fmaxf(fabsf(ndot), expf(-m)) + 1e-6f);
     }
-    if (j_ok && ns == 0) a.y[row * a.y_st + (long)h * a.vdim + j] = yv;
+#pragma unroll
+    for (int c = 0; c < VPT; ++c) {
+      const float d = group_reduce_sum<NSP>(dot[c]);
+      const float yv = KIND == KIND_MLSTM ? d * den : d + c2 * vj[c];
+      if (ns == 0 && jbase + c < a.vdim)
+        a.y[row * a.y_st + (long)h * a.vdim + jbase + c] = yv;
+    }
   }
 
-  if (j_ok) {
+#pragma unroll
+  for (int c = 0; c < VPT; ++c) {
+    if (jbase + c >= a.vdim) continue;
+    float* srow = sbase + (long)(jbase + c) * a.nk;
     if (vec && n0 + NPT <= a.nk) {
 #pragma unroll
       for (int i = 0; i < NPT; i += 4)
         *reinterpret_cast<float4*>(srow + n0 + i) =
-            make_float4(S[i], S[i + 1], S[i + 2], S[i + 3]);
+            make_float4(S[c][i], S[c][i + 1], S[c][i + 2], S[c][i + 3]);
     } else {
 #pragma unroll
       for (int i = 0; i < NPT; ++i)
-        if (n0 + i < a.nk) srow[n0 + i] = S[i];
+        if (n0 + i < a.nk) srow[n0 + i] = S[c][i];
     }
   }
   // the normaliser n and the maximum m are read by every workgroup of this
@@ -233,10 +256,18 @@ void launch_matrix_scan(const ScanArgs& a, int nseq, hipStream_t stream) {
   const int nslices = (a.nk + NPT - 1) / NPT;
   int nsp = 1;
   while (nsp < nslices) nsp <<= 1;
+  // four value columns per thread when that still fills a workgroup: the key
+  // and query slices a thread loads then serve four state columns
 #define SCAN_CASE(P)                                                           \
   case P: {                                                                    \
-    dim3 grid(nseq * a.heads, (a.vdim + 256 / P - 1) / (256 / P));             \
-    matrix_scan_kernel<T, KIND, P><<<grid, 256, 0, stream>>>(a);               \
+    constexpr int JW = 256 / P;                                                \
+    if (a.vdim >= 4 * JW) {                                                    \
+      dim3 grid(nseq * a.heads, (a.vdim + 4 * JW - 1) / (4 * JW));             \
+      matrix_scan_kernel<T, KIND, P, 4><<<grid, 256, 0, stream>>>(a);          \
+    } else {                                                                   \
+      dim3 grid(nseq * a.heads, (a.vdim + JW - 1) / JW);                       \
+      matrix_scan_kernel<T, KIND, P, 1><<<grid, 256, 0, stream>>>(a);          \
+    }                                                                          \
     break;                                                                     \
   }
   switch (nsp) {

@@ -194,7 +194,8 @@ def test_conv_bias_act_slice(dtype, taps):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("sizes", [(4, 24, 16, 2), (3, 20, 40, 1), (2, 64, 128, 1), (5, 8, 6, 5)])
+@pytest.mark.parametrize("sizes", [(4, 24, 16, 2), (3, 20, 40, 1), (2, 64, 128, 1), (5, 8, 6, 5), (2, 160, 128, 2),
+                                   (1, 264, 24, 1)])
 def test_ssd_scan(dtype, sizes):
     heads, vdim, nstate, groups = sizes
     g = torch.Generator().manual_seed(6)
@@ -219,7 +220,7 @@ def test_ssd_scan(dtype, sizes):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("sizes", [(3, 16, 24), (2, 40, 20), (1, 128, 64), (4, 8, 136)])
+@pytest.mark.parametrize("sizes", [(3, 16, 24), (2, 40, 20), (1, 128, 64), (4, 8, 136), (1, 256, 72), (2, 64, 256)])
 def test_mlstm_scan(dtype, sizes):
     heads, dim, vdim = sizes
     g = torch.Generator().manual_seed(7)
