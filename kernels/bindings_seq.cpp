@@ -8,7 +8,7 @@
 #include <hip/hip_bf16.h>
 
 template <typename T>
-void launch_gelu_tanh(T*, const T*, const T*, long, int, long, hipStream_t);
+void launch_gelu_tanh(T*, const T*, long, const T*, long, int, long, hipStream_t);
 template <typename T>
 void launch_embedding_scaled(float*, const long*, const T*, float, int, int,
                              hipStream_t);
@@ -92,9 +92,12 @@ void check_i64(const torch::Tensor& t, const char* what) {
 
 void gelu_tanh(torch::Tensor out, torch::Tensor x,
                c10::optional<torch::Tensor> mul) {
-  TORCH_CHECK(x.is_cuda() && x.is_contiguous() && out.is_contiguous());
+  // x: contiguous of any rank, or a 2-D column slice (rows strided)
+  TORCH_CHECK(x.is_cuda() && out.is_contiguous() &&
+              (x.is_contiguous() || (x.dim() == 2 && x.stride(1) == 1)));
   TORCH_CHECK(out.scalar_type() == x.scalar_type() && out.numel() == x.numel());
   const int cols = x.size(-1);
+  const long x_stride = x.is_contiguous() ? cols : (long)x.stride(0);
   long mul_stride = 0;
   if (mul.has_value()) {
     const auto& m = mul.value();
@@ -105,7 +108,7 @@ void gelu_tanh(torch::Tensor out, torch::Tensor x,
   }
   DISPATCH_F32_BF16(x.scalar_type(), {
     launch_gelu_tanh<scalar_t>(
-        ptr<scalar_t>(out), ptr<scalar_t>(x),
+        ptr<scalar_t>(out), ptr<scalar_t>(x), x_stride,
         mul.has_value() ? ptr<scalar_t>(mul.value()) : nullptr, mul_stride,
         cols, x.numel(), stream());
   });

@@ -308,6 +308,112 @@ __global__ __launch_bounds__(256) void qk_norm_cache_write_kernel(
     dst[c] = ScalarOps<T>::from_f32(ScalarOps<T>::to_f32(src[c]) * f * w[c]);
 }
 
+// Vector variant of gated_group_norm: gsize % 4 == 0, the part held in
+// registers (gsize <= blockDim * 4 * NCH), every input read once.
+template <typename T, int NCH>
+__global__ __launch_bounds__(256) void gated_group_norm_reg_kernel(
+    T* __restrict__ out, const float* __restrict__ y, const T* __restrict__ gate,
+    long gate_stride, const float* __restrict__ w, float eps, int cols, int gsize,
+    int gate_first) {
+  __shared__ float r0[16];
+  const long row = blockIdx.x;
+  const int c0 = blockIdx.y * gsize;
+  const float* yr = y + row * cols + c0;
+  const T* gr = gate + row * gate_stride + c0;
+  float4 v[NCH], sg[NCH];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    const int c = (threadIdx.x + i * blockDim.x) * 4;
+    v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    sg[i] = v[i];
+    if (c < gsize) {
+      v[i] = ld4<float>(yr + c);
+      const float4 g = ld4<T>(gr + c);
+      sg[i] = make_float4(1.0f / (1.0f + expf(-g.x)), 1.0f / (1.0f + expf(-g.y)),
+                          1.0f / (1.0f + expf(-g.z)), 1.0f / (1.0f + expf(-g.w)));
+      if (gate_first) {
+        v[i].x *= g.x * sg[i].x; v[i].y *= g.y * sg[i].y;
+        v[i].z *= g.z * sg[i].z; v[i].w *= g.w * sg[i].w;
+      }
+      ss += (v[i].x * v[i].x + v[i].y * v[i].y) + (v[i].z * v[i].z + v[i].w * v[i].w);
+    }
+  }
+  const float inv = 1.0f / sqrtf(reduce_sum(ss, r0) / gsize + eps);
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    const int c = (threadIdx.x + i * blockDim.x) * 4;
+    if (c < gsize) {
+      const float4 ww = ld4<float>(w + c0 + c);
+      float4 o = make_float4(v[i].x * inv * ww.x, v[i].y * inv * ww.y,
+                             v[i].z * inv * ww.z, v[i].w * inv * ww.w);
+      if (!gate_first) { o.x *= sg[i].x; o.y *= sg[i].y; o.z *= sg[i].z; o.w *= sg[i].w; }
+      st4<T>(out + row * cols + c0 + c, o);
+    }
+  }
+}
+
+// Vector variant of qk_norm_cache_write: 16 lanes per (token, unit), 16-byte
+// accesses; dim, vdim and the row strides are multiples of the vector length.
+template <typename T>
+__global__ __launch_bounds__(256) void qk_norm_cache_write_vec_kernel(
+    T* __restrict__ q_out, const T* __restrict__ q, long q_st,
+    const T* __restrict__ k, long k_st, const T* __restrict__ v, long v_st,
+    const float* __restrict__ qw, const float* __restrict__ kw, float eps,
+    const long* __restrict__ positions, float temp_coef, int temp_every,
+    T* __restrict__ k_cache, T* __restrict__ v_cache,
+    const long* __restrict__ slot_mapping, int heads, int kv_heads, int dim,
+    int vdim) {
+  constexpr int E = Vec16<T>::kElems;
+  constexpr int LPU = 16;
+  const long t = blockIdx.x;
+  const int lane = threadIdx.x % LPU;
+  const int unit = blockIdx.y * (256 / LPU) + threadIdx.x / LPU;
+  if (unit >= heads + 2 * kv_heads) return;   // whole 16-lane groups leave together
+  const long slot = slot_mapping[t];
+  if (unit >= heads + kv_heads) {
+    if (slot < 0) return;
+    const int g = unit - heads - kv_heads;
+    const T* src = v + t * v_st + (long)g * vdim;
+    T* dst = v_cache + (slot * kv_heads + g) * vdim;
+    for (int c = lane * E; c < vdim; c += LPU * E) store16(dst + c, load16(src + c));
+    return;
+  }
+  const bool is_q = unit < heads;
+  const int hh = is_q ? unit : unit - heads;
+  if (!is_q && slot < 0) return;
+  const T* src = is_q ? q + t * q_st + (long)hh * dim : k + t * k_st + (long)hh * dim;
+  float ss = 0.f;
+  for (int c = lane * E; c < dim; c += LPU * E) {
+    const Vec16<T> x = load16(src + c);
+#pragma unroll
+    for (int u = 0; u < E; ++u) {
+      const float f = ScalarOps<T>::to_f32(x.data[u]);
+      ss += f * f;
+    }
+  }
+  ss = group_reduce_sum<LPU>(ss);
+  float f = 1.0f / sqrtf(ss / dim + eps);
+  const float* w = is_q ? qw : kw;
+  T* dst;
+  if (is_q) {
+    if (temp_every > 0) {
+      const long p = positions[t];
+      f *= 1.0f + temp_coef * logf((float)((p + 1) / temp_every) + 1.0f);
+    }
+    dst = q_out + (t * heads + hh) * dim;
+  } else {
+    dst = k_cache + (slot * kv_heads + hh) * dim;
+  }
+  for (int c = lane * E; c < dim; c += LPU * E) {
+    Vec16<T> x = load16(src + c);
+#pragma unroll
+    for (int u = 0; u < E; ++u)
+      x.data[u] = ScalarOps<T>::from_f32(ScalarOps<T>::to_f32(x.data[u]) * f * w[c + u]);
+    store16(dst + c, x);
+  }
+}
+
 template <typename P>
 inline bool al16(const P* p) {   // 8 bytes are enough for 4 bf16, 16 for 4 f32
   return p == nullptr || reinterpret_cast<uintptr_t>(p) % 16 == 0;
@@ -368,8 +474,20 @@ void launch_gated_group_norm(T* out, const float* y, const T* gate,
                              int rows, int cols, int groups, int gate_first,
                              hipStream_t s) {
   const int gsize = cols / groups;
-  const int block = gsize <= 64 ? 64 : (gsize <= 128 ? 128 : 256);
   dim3 grid(rows, groups);
+  if (gsize % 4 == 0 && gate_stride % 4 == 0 && gsize <= 4096 && al16(out) &&
+      al16(y) && al16(gate) && al16(w)) {
+    const int q4 = gsize / 4;
+    const int vb = q4 <= 64 ? 64 : (q4 <= 128 ? 128 : 256);
+    if (q4 <= vb)
+      gated_group_norm_reg_kernel<T, 1><<<grid, vb, 0, s>>>(out, y, gate, gate_stride, w,
+                                                           eps, cols, gsize, gate_first);
+    else
+      gated_group_norm_reg_kernel<T, 4><<<grid, vb, 0, s>>>(out, y, gate, gate_stride, w,
+                                                           eps, cols, gsize, gate_first);
+    return;
+  }
+  const int block = gsize <= 64 ? 64 : (gsize <= 128 ? 128 : 256);
   gated_group_norm_kernel<T><<<grid, block, 0, s>>>(out, y, gate, gate_stride, w, eps,
                                                    cols, gsize, gate_first);
 }
@@ -383,6 +501,16 @@ void launch_qk_norm_cache_write(T* q_out, const T* q, long q_st, const T* k,
                                 int heads, int kv_heads, int dim, int vdim,
                                 hipStream_t s) {
   const int units = heads + 2 * kv_heads;
+  const int e = 16 / sizeof(T);
+  if (dim % e == 0 && vdim % e == 0 && q_st % e == 0 && k_st % e == 0 &&
+      v_st % e == 0 && al16(q_out) && al16(q) && al16(k) && al16(v) &&
+      al16(k_cache) && al16(v_cache)) {
+    dim3 vgrid(tokens, (units + 15) / 16);
+    qk_norm_cache_write_vec_kernel<T><<<vgrid, 256, 0, s>>>(
+        q_out, q, q_st, k, k_st, v, v_st, qw, kw, eps, positions, temp_coef,
+        temp_every, k_cache, v_cache, slot_mapping, heads, kv_heads, dim, vdim);
+    return;
+  }
   dim3 grid(tokens, (units + 3) / 4);
   qk_norm_cache_write_kernel<T><<<grid, 256, 0, s>>>(
       q_out, q, q_st, k, k_st, v, v_st, qw, kw, eps, positions, temp_coef,

@@ -256,7 +256,7 @@ void launch_matrix_scan(const ScanArgs& a, int nseq, hipStream_t stream) {
   const int nslices = (a.nk + NPT - 1) / NPT;
   int nsp = 1;
   while (nsp < nslices) nsp <<= 1;
-  // four value columns per thread when that still fills a workgroup: the key
+  // four (or two) value columns per thread when that still fills a workgroup: the key
   // and query slices a thread loads then serve four state columns
 #define SCAN_CASE(P)                                                           \
   case P: {                                                                    \
@@ -264,6 +264,9 @@ void launch_matrix_scan(const ScanArgs& a, int nseq, hipStream_t stream) {
     if (a.vdim >= 4 * JW) {                                                    \
       dim3 grid(nseq * a.heads, (a.vdim + 4 * JW - 1) / (4 * JW));             \
       matrix_scan_kernel<T, KIND, P, 4><<<grid, 256, 0, stream>>>(a);          \
+    } else if (a.vdim >= 2 * JW) {                                             \
+      dim3 grid(nseq * a.heads, (a.vdim + 2 * JW - 1) / (2 * JW));             \
+      matrix_scan_kernel<T, KIND, P, 2><<<grid, 256, 0, stream>>>(a);          \
     } else {                                                                   \
       dim3 grid(nseq * a.heads, (a.vdim + JW - 1) / JW);                       \
       matrix_scan_kernel<T, KIND, P, 1><<<grid, 256, 0, stream>>>(a);          \

@@ -45,33 +45,31 @@ DEVINLINE float gelu_tanh_f32(float z) {
   return 0.5f * z * (1.0f + tanhf(k * (z + 0.044715f * z * z * z)));
 }
 
-// out = gelu_tanh(x) [* mul]; mul rows may be strided (a column slice).
-// VEC: cols and mul_stride are multiples of 4, n counts groups of 4.
+// out = gelu_tanh(x) [* mul]; x and mul rows may be strided (column slices).
+// VEC: cols and the strides are multiples of 4, n counts groups of 4.
 template <typename T, bool VEC>
 __global__ void gelu_tanh_kernel(T* __restrict__ out, const T* __restrict__ x,
-                                 const T* __restrict__ mul, long mul_stride,
-                                 int cols, long n) {
+                                 long x_stride, const T* __restrict__ mul,
+                                 long mul_stride, int cols, long n) {
   for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < n;
        i += (long)gridDim.x * blockDim.x) {
     if (VEC) {
       const long e = i * 4;
-      F4 f = Pack4<T>::load(x + e);
+      const long r = e / cols;
+      F4 f = Pack4<T>::load(x + r * x_stride + (e - r * cols));
 #pragma unroll
       for (int k = 0; k < 4; ++k) f.v[k] = gelu_tanh_f32(f.v[k]);
       if (mul != nullptr) {
-        const long r = e / cols;
         const F4 m = Pack4<T>::load(mul + r * mul_stride + (e - r * cols));
 #pragma unroll
         for (int k = 0; k < 4; ++k) f.v[k] *= m.v[k];
       }
       Pack4<T>::store(out + e, f);
     } else {
-      float y = gelu_tanh_f32(ScalarOps<T>::to_f32(x[i]));
-      if (mul != nullptr) {
-        const long r = i / cols;
-        const int c = (int)(i - r * cols);
-        y *= ScalarOps<T>::to_f32(mul[r * mul_stride + c]);
-      }
+      const long r = i / cols;
+      const int c = (int)(i - r * cols);
+      float y = gelu_tanh_f32(ScalarOps<T>::to_f32(x[r * x_stride + c]));
+      if (mul != nullptr) y *= ScalarOps<T>::to_f32(mul[r * mul_stride + c]);
       out[i] = ScalarOps<T>::from_f32(y);
     }
   }
@@ -307,13 +305,15 @@ static inline int grid_for(long n, int block) {
 }
 
 template <typename T>
-void launch_gelu_tanh(T* out, const T* x, const T* mul, long mul_stride,
-                      int cols, long n, hipStream_t s) {
-  if (cols % 4 == 0 && mul_stride % 4 == 0 && al(out, 4 * sizeof(T)) &&
-      al(x, 4 * sizeof(T)) && al(mul, 4 * sizeof(T)))
-    gelu_tanh_kernel<T, true><<<grid_for(n / 4, 256), 256, 0, s>>>(out, x, mul, mul_stride, cols, n / 4);
+void launch_gelu_tanh(T* out, const T* x, long x_stride, const T* mul,
+                      long mul_stride, int cols, long n, hipStream_t s) {
+  if (cols % 4 == 0 && mul_stride % 4 == 0 && x_stride % 4 == 0 &&
+      al(out, 4 * sizeof(T)) && al(x, 4 * sizeof(T)) && al(mul, 4 * sizeof(T)))
+    gelu_tanh_kernel<T, true><<<grid_for(n / 4, 256), 256, 0, s>>>(
+        out, x, x_stride, mul, mul_stride, cols, n / 4);
   else
-    gelu_tanh_kernel<T, false><<<grid_for(n, 256), 256, 0, s>>>(out, x, mul, mul_stride, cols, n);
+    gelu_tanh_kernel<T, false><<<grid_for(n, 256), 256, 0, s>>>(
+        out, x, x_stride, mul, mul_stride, cols, n);
 }
 template <typename T>
 void launch_embedding_scaled(float* out, const long* ids, const T* table,
@@ -372,8 +372,8 @@ void launch_latent_kv_write(const T* dkv, const float* norm_w, float eps,
 }
 
 #define INSTANTIATE(T)                                                          \
-  template void launch_gelu_tanh<T>(T*, const T*, const T*, long, int, long,    \
-                                    hipStream_t);                               \
+  template void launch_gelu_tanh<T>(T*, const T*, long, const T*, long, int,    \
+                                    long, hipStream_t);                         \
   template void launch_embedding_scaled<T>(float*, const long*, const T*,       \
                                            float, int, int, hipStream_t);       \
   template void launch_rms_norm_stream<T>(T*, const float*, const float*,       \

@@ -36,7 +36,7 @@ def _seqs(spec):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("width", [96, 250])
+@pytest.mark.parametrize("width", [96, 250, 1024, 2052, 5120, 9000])
 def test_layer_norms(dtype, width):
     g = torch.Generator().manual_seed(1)
     x = torch.randn(7, width, generator=g) * 3 + 1
@@ -79,10 +79,20 @@ def test_gated_group_norm(dtype, gate_first):
                                    1e-5, gate_first, dtype)
         _close(out, ref.gated_group_norm(y, gate, w, groups, 1e-5, gate_first, dtype),
                dtype, f"groups {groups}")
+    # 16-byte paths: aligned gate slice, parts of 64 to 4096 values, and 6144
+    y = torch.randn(3, 6144, generator=g)
+    wide = torch.randn(3, 6144 + 128, generator=g).to(dtype)
+    w = torch.rand(6144, generator=g) + 0.5
+    for groups in (96, 12, 3, 2, 1):
+        out = ops.gated_group_norm(y.to(DEV), wide.to(DEV)[:, 64:64 + 6144], w.to(DEV), groups,
+                                   1e-5, gate_first, dtype)
+        _close(out, ref.gated_group_norm(y, wide[:, 64:64 + 6144], w, groups, 1e-5, gate_first,
+                                         dtype), dtype, f"wide groups {groups}")
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("dims", [(5, 5, 24, 40), (6, 2, 32, 32), (4, 1, 72, 16)])
+@pytest.mark.parametrize("dims", [(5, 5, 24, 40), (6, 2, 32, 32), (4, 1, 72, 16), (3, 3, 10, 6),
+                                  (8, 2, 128, 128), (2, 1, 256, 64)])
 def test_qk_norm_and_attention(dtype, dims):
     heads, kvh, dim, vdim = dims
     g = torch.Generator().manual_seed(3)

@@ -267,7 +267,7 @@ class GatedDenseMLP(nn.Module):
 
     def forward(self, h: torch.Tensor) -> torch.Tensor:
         gu = ops.linear(h, self.gate_up)
-        a = ops.gelu_tanh(gu[:, :self.ff].contiguous(), mul=gu[:, self.ff:])
+        a = ops.gelu_tanh(gu[:, :self.ff], mul=gu[:, self.ff:])
         return ops.linear(a, self.down)
 
 
@@ -488,7 +488,7 @@ class RGLRUMixer(_Mixer):
     def mix(self, proj, positions, cache, meta: AttnMetadata) -> torch.Tensor:
         conv_state, rec_state = cache
         t, w, nb = proj.shape[0], self.rec_width, self.blocks
-        yb = ops.gelu_tanh(proj[:, :w].contiguous())
+        yb = ops.gelu_tanh(proj[:, :w])
         u = ops.causal_conv_state(
             proj[:, w:], self.conv_weight, conv_state, meta.seq_start_loc,
             meta.seq_lens, meta.state_slots, add_input=False, bias=self.conv_bias)

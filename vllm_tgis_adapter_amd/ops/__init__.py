@@ -456,9 +456,10 @@ def _native_seq(t: torch.Tensor) -> bool:
 
 
 def gelu_tanh(x: torch.Tensor, mul: torch.Tensor | None = None) -> torch.Tensor:
-    """tanh-form GELU, optionally times ``mul`` (rows may be strided)."""
+    """tanh-form GELU, optionally times ``mul``; x and mul may be column
+    slices of a wider matrix (strided rows)."""
     if x.numel() and _native_seq(x):
-        out = torch.empty_like(x)
+        out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
         _S.gelu_tanh(out, x, mul)
         return out
     return reference.gelu_tanh(x, mul)
