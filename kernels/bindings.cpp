@@ -93,6 +93,9 @@ void launch_moe_gemm(__hip_bfloat16*, const __hip_bfloat16*,
                      const __hip_bfloat16*, const int*, int, int, int, int,
                      bool, hipStream_t);
 
+// paged attention (bindings_attn.cpp, shared with the `_C_attn` extension)
+void register_attention_ops(pybind11::module& m);
+
 namespace {
 
 hipStream_t current_stream() {
@@ -203,140 +206,6 @@ void reshape_and_cache(torch::Tensor k, torch::Tensor v, torch::Tensor k_cache,
         cptr<scalar_t>(k), cptr<scalar_t>(v), ptr<scalar_t>(k_cache),
         ptr<scalar_t>(v_cache), slot_mapping.data_ptr<long>(), tokens,
         row_elems, current_stream());
-  });
-}
-
-void paged_attention_decode(torch::Tensor out, torch::Tensor q,
-                            torch::Tensor k_cache, torch::Tensor v_cache,
-                            torch::Tensor block_tables, torch::Tensor seq_lens,
-                            double scale) {
-  const int nseq = q.size(0);
-  const int nheads = q.size(1);
-  const int head_dim = q.size(2);
-  const int kvh = k_cache.size(2);
-  const int block_size = k_cache.size(1);
-  const int max_blocks = block_tables.size(1);
-  TORCH_CHECK(block_tables.scalar_type() == at::ScalarType::Int);
-  TORCH_CHECK(seq_lens.scalar_type() == at::ScalarType::Int);
-  const int group = nheads / kvh;
-  static const bool force_valu = [] {
-    const char* e = getenv("VTA_DECODE_VALU");
-    return e && e[0] == '1';
-  }();
-  const bool kv_fp8 = k_cache.scalar_type() == at::ScalarType::Byte;
-  if (kv_fp8) {
-    TORCH_CHECK(q.scalar_type() == at::ScalarType::BFloat16 &&
-                    (head_dim == 64 || head_dim == 128) && group >= 1 &&
-                    group <= 8,
-                "fp8 KV cache requires the bf16 MFMA decode path");
-    const int npart = decode_mfma_num_partitions(nseq, kvh, max_blocks * block_size);
-    const int P = npart * 4;
-    auto opts = q.options().dtype(at::ScalarType::Float);
-    auto part_acc = at::empty({nseq, nheads, P, head_dim}, opts);
-    auto part_ml = at::empty({nseq, nheads, P, 2}, opts);
-    launch_paged_decode_mfma_fp8(
-        reinterpret_cast<__hip_bfloat16*>(out.data_ptr()),
-        part_acc.data_ptr<float>(), part_ml.data_ptr<float>(),
-        reinterpret_cast<const __hip_bfloat16*>(q.data_ptr()),
-        reinterpret_cast<const unsigned char*>(k_cache.data_ptr()),
-        reinterpret_cast<const unsigned char*>(v_cache.data_ptr()),
-        block_tables.data_ptr<int>(), seq_lens.data_ptr<int>(), (float)scale,
-        nseq, nheads, kvh, head_dim, block_size, max_blocks, npart,
-        current_stream());
-    return;
-  }
-  if (!force_valu && q.scalar_type() == at::ScalarType::BFloat16 &&
-      (head_dim == 64 || head_dim == 128) && group >= 1 && group <= 8 &&
-      nheads == kvh * group && nseq > 0) {
-    const int npart = decode_mfma_num_partitions(nseq, kvh, max_blocks * block_size);
-    const int P = npart * 4;
-    auto opts = q.options().dtype(at::ScalarType::Float);
-    auto part_acc = at::empty({nseq, nheads, P, head_dim}, opts);
-    auto part_ml = at::empty({nseq, nheads, P, 2}, opts);
-    launch_paged_decode_mfma(
-        reinterpret_cast<__hip_bfloat16*>(out.data_ptr()),
-        part_acc.data_ptr<float>(), part_ml.data_ptr<float>(),
-        reinterpret_cast<const __hip_bfloat16*>(q.data_ptr()),
-        reinterpret_cast<const __hip_bfloat16*>(k_cache.data_ptr()),
-        reinterpret_cast<const __hip_bfloat16*>(v_cache.data_ptr()),
-        block_tables.data_ptr<int>(), seq_lens.data_ptr<int>(), (float)scale,
-        nseq, nheads, kvh, head_dim, block_size, max_blocks, npart,
-        current_stream());
-    return;
-  }
-  DISPATCH_FLOATING(q.scalar_type(), {
-    launch_paged_decode<scalar_t>(
-        ptr<scalar_t>(out), cptr<scalar_t>(q), cptr<scalar_t>(k_cache),
-        cptr<scalar_t>(v_cache), block_tables.data_ptr<int>(),
-        seq_lens.data_ptr<int>(), (float)scale, nseq, nheads, kvh, head_dim,
-        block_size, max_blocks, current_stream());
-  });
-}
-
-void paged_attention_prefill(torch::Tensor out, torch::Tensor q,
-                             torch::Tensor k_cache, torch::Tensor v_cache,
-                             torch::Tensor block_tables,
-                             torch::Tensor query_start_loc,
-                             torch::Tensor seq_lens, double scale,
-                             int64_t max_query_len) {
-  const int nseq = seq_lens.size(0);
-  const int nheads = q.size(1);
-  const int head_dim = q.size(2);
-  const int kvh = k_cache.size(2);
-  const int block_size = k_cache.size(1);
-  const int max_blocks = block_tables.size(1);
-  static const bool force_valu = [] {
-    const char* e = getenv("VTA_PREFILL_VALU");
-    return e && e[0] == '1';
-  }();
-  static const bool force_v1 = [] {
-    const char* e = getenv("VTA_PREFILL_V1");
-    return e && e[0] == '1';
-  }();
-  if (k_cache.scalar_type() == at::ScalarType::Byte) {
-    TORCH_CHECK(q.scalar_type() == at::ScalarType::BFloat16 && head_dim == 128,
-                "fp8 KV cache requires the bf16 v2 prefill path (hd=128)");
-    launch_paged_prefill_mfma_v2_fp8(
-        reinterpret_cast<__hip_bfloat16*>(out.data_ptr()),
-        reinterpret_cast<const __hip_bfloat16*>(q.data_ptr()),
-        reinterpret_cast<const unsigned char*>(k_cache.data_ptr()),
-        reinterpret_cast<const unsigned char*>(v_cache.data_ptr()),
-        block_tables.data_ptr<int>(), query_start_loc.data_ptr<int>(),
-        seq_lens.data_ptr<int>(), (float)scale, nseq, nheads, kvh, head_dim,
-        block_size, max_blocks, (int)max_query_len, current_stream());
-    return;
-  }
-  if (!force_valu && !force_v1 &&
-      q.scalar_type() == at::ScalarType::BFloat16 && head_dim == 128) {
-    launch_paged_prefill_mfma_v2(
-        reinterpret_cast<__hip_bfloat16*>(out.data_ptr()),
-        reinterpret_cast<const __hip_bfloat16*>(q.data_ptr()),
-        reinterpret_cast<const __hip_bfloat16*>(k_cache.data_ptr()),
-        reinterpret_cast<const __hip_bfloat16*>(v_cache.data_ptr()),
-        block_tables.data_ptr<int>(), query_start_loc.data_ptr<int>(),
-        seq_lens.data_ptr<int>(), (float)scale, nseq, nheads, kvh, head_dim,
-        block_size, max_blocks, (int)max_query_len, current_stream());
-    return;
-  }
-  if (!force_valu && q.scalar_type() == at::ScalarType::BFloat16 &&
-      (head_dim == 64 || head_dim == 128)) {
-    launch_paged_prefill_mfma(
-        reinterpret_cast<__hip_bfloat16*>(out.data_ptr()),
-        reinterpret_cast<const __hip_bfloat16*>(q.data_ptr()),
-        reinterpret_cast<const __hip_bfloat16*>(k_cache.data_ptr()),
-        reinterpret_cast<const __hip_bfloat16*>(v_cache.data_ptr()),
-        block_tables.data_ptr<int>(), query_start_loc.data_ptr<int>(),
-        seq_lens.data_ptr<int>(), (float)scale, nseq, nheads, kvh, head_dim,
-        block_size, max_blocks, (int)max_query_len, current_stream());
-    return;
-  }
-  DISPATCH_FLOATING(q.scalar_type(), {
-    launch_paged_prefill<scalar_t>(
-        ptr<scalar_t>(out), cptr<scalar_t>(q), cptr<scalar_t>(k_cache),
-        cptr<scalar_t>(v_cache), block_tables.data_ptr<int>(),
-        query_start_loc.data_ptr<int>(), seq_lens.data_ptr<int>(),
-        (float)scale, nseq, nheads, kvh, head_dim, block_size, max_blocks,
-        (int)max_query_len, current_stream());
   });
 }
 
@@ -590,10 +459,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("silu_and_mul", &silu_and_mul, "SwiGLU activation (CDNA4)");
   m.def("rotary_embedding", &rotary_embedding, "NeoX rotary, in place (CDNA4)");
   m.def("reshape_and_cache", &reshape_and_cache, "paged KV cache write (CDNA4)");
-  m.def("paged_attention_decode", &paged_attention_decode,
-        "paged decode attention (CDNA4)");
-  m.def("paged_attention_prefill", &paged_attention_prefill,
-        "paged causal prefill attention (CDNA4)");
+  register_attention_ops(m);
   m.def("xar_alloc", &xar_alloc,
         "raw hipMalloc + IPC handle for the xGMI all-reduce staging buffer");
   m.def("xar_open", &xar_open, "open a peer's IPC handle -> device pointer");

@@ -1,0 +1,223 @@
+// Torch bindings of the paged grouped-query attention kernels (generic f32 /
+// f16 / bf16, bf16 MFMA decode and prefill, fp8 cache variants).  Compiled
+// into `_C` and, with module_attn.cpp, into the small `_C_attn` extension for
+// models that need nothing else of `_C`.
+
+#include <torch/extension.h>
+#include <ATen/hip/HIPContext.h>
+
+#include <hip/hip_bf16.h>
+#include <hip/hip_fp16.h>
+
+template <typename T>
+void launch_paged_decode(T*, const T*, const T*, const T*, const int*,
+                         const int*, float, int, int, int, int, int, int,
+                         hipStream_t);
+template <typename T>
+void launch_paged_prefill(T*, const T*, const T*, const T*, const int*,
+                          const int*, const int*, float, int, int, int, int,
+                          int, int, int, hipStream_t);
+void launch_paged_prefill_mfma_v2(__hip_bfloat16*, const __hip_bfloat16*,
+                                  const __hip_bfloat16*, const __hip_bfloat16*,
+                                  const int*, const int*, const int*, float,
+                                  int, int, int, int, int, int, int,
+                                  hipStream_t);
+void launch_paged_prefill_mfma(__hip_bfloat16*, const __hip_bfloat16*,
+                               const __hip_bfloat16*, const __hip_bfloat16*,
+                               const int*, const int*, const int*, float, int,
+                               int, int, int, int, int, int, hipStream_t);
+int decode_mfma_num_partitions(int nseq, int kvh, int max_context);
+void launch_paged_decode_mfma_fp8(__hip_bfloat16*, float*, float*,
+                                  const __hip_bfloat16*, const unsigned char*,
+                                  const unsigned char*, const int*,
+                                  const int*, float, int, int, int, int, int,
+                                  int, int, hipStream_t);
+void launch_paged_prefill_mfma_v2_fp8(__hip_bfloat16*, const __hip_bfloat16*,
+                                      const unsigned char*,
+                                      const unsigned char*, const int*,
+                                      const int*, const int*, float, int, int,
+                                      int, int, int, int, int, hipStream_t);
+void launch_paged_decode_mfma(__hip_bfloat16*, float*, float*,
+                              const __hip_bfloat16*, const __hip_bfloat16*,
+                              const __hip_bfloat16*, const int*, const int*,
+                              float, int, int, int, int, int, int, int,
+                              hipStream_t);
+
+namespace {
+
+hipStream_t current_stream() {
+  return at::hip::getCurrentHIPStream().stream();
+}
+
+template <typename T>
+T* ptr(torch::Tensor& t) {
+  return reinterpret_cast<T*>(t.data_ptr());
+}
+template <typename T>
+const T* cptr(const torch::Tensor& t) {
+  return reinterpret_cast<const T*>(t.data_ptr());
+}
+
+#define DISPATCH_FLOATING(DTYPE, BODY)                                   \
+  switch (DTYPE) {                                                       \
+    case at::ScalarType::BFloat16: {                                     \
+      using scalar_t = __hip_bfloat16;                                   \
+      BODY;                                                              \
+      break;                                                             \
+    }                                                                    \
+    case at::ScalarType::Half: {                                         \
+      using scalar_t = __half;                                           \
+      BODY;                                                              \
+      break;                                                             \
+    }                                                                    \
+    case at::ScalarType::Float: {                                        \
+      using scalar_t = float;                                            \
+      BODY;                                                              \
+      break;                                                             \
+    }                                                                    \
+    default:                                                             \
+      TORCH_CHECK(false, "unsupported dtype");                           \
+  }
+
+void paged_attention_decode(torch::Tensor out, torch::Tensor q,
+                            torch::Tensor k_cache, torch::Tensor v_cache,
+                            torch::Tensor block_tables, torch::Tensor seq_lens,
+                            double scale) {
+  const int nseq = q.size(0);
+  const int nheads = q.size(1);
+  const int head_dim = q.size(2);
+  const int kvh = k_cache.size(2);
+  const int block_size = k_cache.size(1);
+  const int max_blocks = block_tables.size(1);
+  TORCH_CHECK(block_tables.scalar_type() == at::ScalarType::Int);
+  TORCH_CHECK(seq_lens.scalar_type() == at::ScalarType::Int);
+  const int group = nheads / kvh;
+  static const bool force_valu = [] {
+    const char* e = getenv("VTA_DECODE_VALU");
+    return e && e[0] == '1';
+  }();
+  const bool kv_fp8 = k_cache.scalar_type() == at::ScalarType::Byte;
+  if (kv_fp8) {
+    TORCH_CHECK(q.scalar_type() == at::ScalarType::BFloat16 &&
+                    (head_dim == 64 || head_dim == 128) && group >= 1 &&
+                    group <= 8,
+                "fp8 KV cache requires the bf16 MFMA decode path");
+    const int npart = decode_mfma_num_partitions(nseq, kvh, max_blocks * block_size);
+    const int P = npart * 4;
+    auto opts = q.options().dtype(at::ScalarType::Float);
+    auto part_acc = at::empty({nseq, nheads, P, head_dim}, opts);
+    auto part_ml = at::empty({nseq, nheads, P, 2}, opts);
+    launch_paged_decode_mfma_fp8(
+        reinterpret_cast<__hip_bfloat16*>(out.data_ptr()),
+        part_acc.data_ptr<float>(), part_ml.data_ptr<float>(),
+        reinterpret_cast<const __hip_bfloat16*>(q.data_ptr()),
+        reinterpret_cast<const unsigned char*>(k_cache.data_ptr()),
+        reinterpret_cast<const unsigned char*>(v_cache.data_ptr()),
+        block_tables.data_ptr<int>(), seq_lens.data_ptr<int>(), (float)scale,
+        nseq, nheads, kvh, head_dim, block_size, max_blocks, npart,
+        current_stream());
+    return;
+  }
+  if (!force_valu && q.scalar_type() == at::ScalarType::BFloat16 &&
+      (head_dim == 64 || head_dim == 128) && group >= 1 && group <= 8 &&
+      nheads == kvh * group && nseq > 0) {
+    const int npart = decode_mfma_num_partitions(nseq, kvh, max_blocks * block_size);
+    const int P = npart * 4;
+    auto opts = q.options().dtype(at::ScalarType::Float);
+    auto part_acc = at::empty({nseq, nheads, P, head_dim}, opts);
+    auto part_ml = at::empty({nseq, nheads, P, 2}, opts);
+    launch_paged_decode_mfma(
+        reinterpret_cast<__hip_bfloat16*>(out.data_ptr()),
+        part_acc.data_ptr<float>(), part_ml.data_ptr<float>(),
+        reinterpret_cast<const __hip_bfloat16*>(q.data_ptr()),
+        reinterpret_cast<const __hip_bfloat16*>(k_cache.data_ptr()),
+        reinterpret_cast<const __hip_bfloat16*>(v_cache.data_ptr()),
+        block_tables.data_ptr<int>(), seq_lens.data_ptr<int>(), (float)scale,
+        nseq, nheads, kvh, head_dim, block_size, max_blocks, npart,
+        current_stream());
+    return;
+  }
+  DISPATCH_FLOATING(q.scalar_type(), {
+    launch_paged_decode<scalar_t>(
+        ptr<scalar_t>(out), cptr<scalar_t>(q), cptr<scalar_t>(k_cache),
+        cptr<scalar_t>(v_cache), block_tables.data_ptr<int>(),
+        seq_lens.data_ptr<int>(), (float)scale, nseq, nheads, kvh, head_dim,
+        block_size, max_blocks, current_stream());
+  });
+}
+
+void paged_attention_prefill(torch::Tensor out, torch::Tensor q,
+                             torch::Tensor k_cache, torch::Tensor v_cache,
+                             torch::Tensor block_tables,
+                             torch::Tensor query_start_loc,
+                             torch::Tensor seq_lens, double scale,
+                             int64_t max_query_len) {
+  const int nseq = seq_lens.size(0);
+  const int nheads = q.size(1);
+  const int head_dim = q.size(2);
+  const int kvh = k_cache.size(2);
+  const int block_size = k_cache.size(1);
+  const int max_blocks = block_tables.size(1);
+  static const bool force_valu = [] {
+    const char* e = getenv("VTA_PREFILL_VALU");
+    return e && e[0] == '1';
+  }();
+  static const bool force_v1 = [] {
+    const char* e = getenv("VTA_PREFILL_V1");
+    return e && e[0] == '1';
+  }();
+  if (k_cache.scalar_type() == at::ScalarType::Byte) {
+    TORCH_CHECK(q.scalar_type() == at::ScalarType::BFloat16 && head_dim == 128,
+                "fp8 KV cache requires the bf16 v2 prefill path (hd=128)");
+    launch_paged_prefill_mfma_v2_fp8(
+        reinterpret_cast<__hip_bfloat16*>(out.data_ptr()),
+        reinterpret_cast<const __hip_bfloat16*>(q.data_ptr()),
+        reinterpret_cast<const unsigned char*>(k_cache.data_ptr()),
+        reinterpret_cast<const unsigned char*>(v_cache.data_ptr()),
+        block_tables.data_ptr<int>(), query_start_loc.data_ptr<int>(),
+        seq_lens.data_ptr<int>(), (float)scale, nseq, nheads, kvh, head_dim,
+        block_size, max_blocks, (int)max_query_len, current_stream());
+    return;
+  }
+  if (!force_valu && !force_v1 &&
+      q.scalar_type() == at::ScalarType::BFloat16 && head_dim == 128) {
+    launch_paged_prefill_mfma_v2(
+        reinterpret_cast<__hip_bfloat16*>(out.data_ptr()),
+        reinterpret_cast<const __hip_bfloat16*>(q.data_ptr()),
+        reinterpret_cast<const __hip_bfloat16*>(k_cache.data_ptr()),
+        reinterpret_cast<const __hip_bfloat16*>(v_cache.data_ptr()),
+        block_tables.data_ptr<int>(), query_start_loc.data_ptr<int>(),
+        seq_lens.data_ptr<int>(), (float)scale, nseq, nheads, kvh, head_dim,
+        block_size, max_blocks, (int)max_query_len, current_stream());
+    return;
+  }
+  if (!force_valu && q.scalar_type() == at::ScalarType::BFloat16 &&
+      (head_dim == 64 || head_dim == 128)) {
+    launch_paged_prefill_mfma(
+        reinterpret_cast<__hip_bfloat16*>(out.data_ptr()),
+        reinterpret_cast<const __hip_bfloat16*>(q.data_ptr()),
+        reinterpret_cast<const __hip_bfloat16*>(k_cache.data_ptr()),
+        reinterpret_cast<const __hip_bfloat16*>(v_cache.data_ptr()),
+        block_tables.data_ptr<int>(), query_start_loc.data_ptr<int>(),
+        seq_lens.data_ptr<int>(), (float)scale, nseq, nheads, kvh, head_dim,
+        block_size, max_blocks, (int)max_query_len, current_stream());
+    return;
+  }
+  DISPATCH_FLOATING(q.scalar_type(), {
+    launch_paged_prefill<scalar_t>(
+        ptr<scalar_t>(out), cptr<scalar_t>(q), cptr<scalar_t>(k_cache),
+        cptr<scalar_t>(v_cache), block_tables.data_ptr<int>(),
+        query_start_loc.data_ptr<int>(), seq_lens.data_ptr<int>(),
+        (float)scale, nseq, nheads, kvh, head_dim, block_size, max_blocks,
+        (int)max_query_len, current_stream());
+  });
+}
+
+}  // namespace
+
+void register_attention_ops(pybind11::module& m) {
+  m.def("paged_attention_decode", &paged_attention_decode,
+        "paged decode attention (CDNA4)");
+  m.def("paged_attention_prefill", &paged_attention_prefill,
+        "paged causal prefill attention (CDNA4)");
+}

@@ -5,14 +5,18 @@ kernel sources plus their torch bindings for gfx950 and links the shared
 objects under vllm_tgis_adapter_amd/.  The built .so files travel with the
 repo snapshot to GPU boxes (a JIT cache would not).
 
-Two extensions, so that a model only needs the one it uses:
+Several extensions, so that a model only builds the ones it uses
+(``vllm_tgis_adapter_amd.models.native_extensions`` names them per model):
 
-``_C``    the llama/mixtral/opt kernel set (every kernels/*.hip that is not
-          listed for another extension) + bindings.cpp
-``_C_seq`` f32-residual-stream ops (RMS and layer norms), short causal
-          convolution with per-sequence state, windowed latent attention with
-          sinks, grouped-query attention of any shape, recurrences with
-          per-sequence state + bindings_seq.cpp, bindings_rec.cpp
+``_C``      the llama/mixtral/opt kernel set (every kernels/*.hip that is not
+            listed for another extension) + bindings.cpp, bindings_attn.cpp
+``_C_attn`` only the paged grouped-query attention kernels of ``_C`` (generic
+            and MFMA) + bindings_attn.cpp, module_attn.cpp
+``_C_seq``  f32-residual-stream ops (RMS and layer norms), short causal
+            convolution with per-sequence state, grouped-query attention of
+            any shape, recurrences with per-sequence state + bindings_seq.cpp,
+            bindings_rec.cpp
+``_C_lat``  windowed latent attention with sinks + bindings_lat.cpp
 """
 
 from __future__ import annotations
@@ -29,19 +33,28 @@ KERNELS = REPO / "kernels"
 PKG = REPO / "vllm_tgis_adapter_amd"
 ARCH = os.environ.get("PYTORCH_ROCM_ARCH", "gfx950")
 
-_SEQ_SOURCES = ["stream_ops.hip", "canon_conv.hip", "latent_attention.hip",
-                "latent_attention_mfma.hip", "layer_norm_stream.hip",
+_SEQ_SOURCES = ["stream_ops.hip", "canon_conv.hip", "layer_norm_stream.hip",
                 "paged_attention_any.hip", "recurrent_scan.hip"]
+_LAT_SOURCES = ["latent_attention.hip", "latent_attention_mfma.hip"]
+_ATTN_SOURCES = ["attention.hip", "attention_decode_mfma.hip",
+                 "attention_prefill_mfma.hip", "attention_prefill_mfma_v2.hip"]
 
 EXTENSIONS = {
     "_C": dict(
         sources=lambda: [p for p in sorted(KERNELS.glob("*.hip"))
-                         if p.name not in _SEQ_SOURCES] + [KERNELS / "bindings.cpp"],
+                         if p.name not in _SEQ_SOURCES + _LAT_SOURCES]
+        + [KERNELS / "bindings.cpp", KERNELS / "bindings_attn.cpp"],
+    ),
+    "_C_attn": dict(
+        sources=lambda: [KERNELS / n for n in _ATTN_SOURCES]
+        + [KERNELS / "bindings_attn.cpp", KERNELS / "module_attn.cpp"],
     ),
     "_C_seq": dict(
-        sources=lambda: [KERNELS / n for n in _SEQ_SOURCES
-                         if (KERNELS / n).exists()]
+        sources=lambda: [KERNELS / n for n in _SEQ_SOURCES]
         + [KERNELS / "bindings_seq.cpp", KERNELS / "bindings_rec.cpp"],
+    ),
+    "_C_lat": dict(
+        sources=lambda: [KERNELS / n for n in _LAT_SOURCES] + [KERNELS / "bindings_lat.cpp"],
     ),
 }
 OUT = PKG / "_C.so"
@@ -93,8 +106,12 @@ def build_ext(name: str, verbose: bool = True, force: bool = False) -> Path:
 
     objects = []
     jobs = []
+    # sources holding a PYBIND11_MODULE bake the extension's name in; all
+    # others are shared between extensions as they are
+    module_sources = {"bindings.cpp", "bindings_seq.cpp", "bindings_lat.cpp", "module_attn.cpp"}
     for src in sources:
         obj = build_dir / (src.stem + ".o")
+        assert src.name in module_sources or "TORCH_EXTENSION_NAME" not in src.read_text()
         objects.append(obj)
         if obj.exists() and not force and obj.stat().st_mtime > max(
             src.stat().st_mtime, common_h.stat().st_mtime

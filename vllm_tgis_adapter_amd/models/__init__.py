@@ -34,7 +34,7 @@ def native_extensions(cfg: ModelConfig) -> list[str]:
     model's forward reaches on a GPU — what a fresh checkout has to build
     before it can serve this model."""
     if cfg.architecture == "dolodra":
-        return ["_C_seq"]
+        return ["_C_seq", "_C_lat"]
     if cfg.architecture == "kezunex":
         from .kezunex import native_extensions as kz
 

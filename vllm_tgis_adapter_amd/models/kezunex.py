@@ -123,8 +123,8 @@ def model_config_from_json(model: str, hf: dict) -> ModelConfig:
 
 def native_extensions(cfg: ModelConfig) -> list[str]:
     """The stream / recurrence / any-shape attention kernels always; the
-    llama-class MFMA attention kernels when an attention mixer has a shape
-    they take."""
+    llama-class MFMA attention kernels (alone, without the rest of that
+    extension) when an attention mixer has a shape they take."""
     need = ["_C_seq"]
     for e in cfg.hf_config["layers"]:
         if e.get("type") != "parallel":
@@ -132,7 +132,7 @@ def native_extensions(cfg: ModelConfig) -> list[str]:
         a = e["mixer"]["left"]
         if ops.attention_uses_matrix_cores(cfg.dtype, int(a["heads"]), int(a["kv_heads"]),
                                            int(a["dim"]), int(a["vdim"])):
-            return need + ["_C"]
+            return need + ["_C_attn"]
     return need
 
 

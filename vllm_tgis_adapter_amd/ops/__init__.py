@@ -407,8 +407,9 @@ make_cos_sin_cache = reference.make_cos_sin_cache
 
 # ---------------------------------------------------------------------------
 # `_C_seq`: f32 residual-stream ops, short causal convolution with
-# per-sequence state, windowed latent attention with sinks.  A separate
-# extension so a model that needs only these compiles only these.
+# per-sequence state (further down: layer norms, any-shape attention,
+# recurrences); `_C_lat`: windowed latent attention with sinks.  Separate
+# extensions so a model that needs only these compiles only these.
 # ---------------------------------------------------------------------------
 
 _S = None
@@ -430,10 +431,65 @@ def _try_load_seq() -> None:
 _try_load_seq()
 
 
+_L = None          # `_C_lat`: latent attention
+_A = None          # `_C_attn`: paged attention alone (when `_C` is not built)
+_lat_load_error: str | None = None
+
+
+def _try_load_lat() -> None:
+    global _L, _lat_load_error
+    if _L is not None:
+        return
+    try:
+        from vllm_tgis_adapter_amd import _C_lat as ext
+
+        _L = ext
+    except ImportError as e:
+        _lat_load_error = str(e)
+
+
+def _try_load_attn() -> None:
+    global _A
+    if _A is not None or _C is not None:
+        return
+    try:
+        from vllm_tgis_adapter_amd import _C_attn as ext
+
+        _A = ext
+    except ImportError:
+        pass
+
+
+_try_load_lat()
+_try_load_attn()
+
+
+def _native_lat(t: torch.Tensor) -> bool:
+    if t.device.type != "cuda" or _FORCE_REFERENCE:
+        return False
+    if _L is None:
+        _try_load_lat()
+    if _L is None:
+        raise RuntimeError(
+            "vllm_tgis_adapter_amd._C_lat HIP extension is not built but a GPU "
+            f"tensor reached one of its ops (import error: {_lat_load_error}). "
+            "Run `python kernels/build.py --only=_C_lat` first."
+        )
+    return True
+
+
+def _attn_ext():
+    """The extension that holds the llama-class paged attention kernels: all
+    of ``_C`` when it is built, else the attention-only ``_C_attn``."""
+    return _C if _C is not None else _A
+
+
 def reload_native() -> None:
     """Load extensions that were built after this module was imported."""
     _try_load_native()
     _try_load_seq()
+    _try_load_lat()
+    _try_load_attn()
 
 
 def has_native_seq() -> bool:
@@ -578,8 +634,8 @@ def latent_attention_prefill(q_lat, q_rot, cache, block_tables, query_start_loc,
     for query chunks (the tail rows of each sequence).  bf16 shapes on the
     MFMA kernel's list run there unless ``general`` asks for the any-shape
     kernel (f32 always does)."""
-    if q_lat.numel() and _native_seq(q_lat):
-        _S.latent_attention_prefill(out, q_lat, q_rot, cache, block_tables,
+    if q_lat.numel() and _native_lat(q_lat):
+        _L.latent_attention_prefill(out, q_lat, q_rot, cache, block_tables,
                                     query_start_loc, seq_lens, float(scale),
                                     int(window), sinks, int(max_query_len), bool(general))
         return out
@@ -593,8 +649,8 @@ def latent_attention_decode(q_lat, q_rot, cache, block_tables, seq_lens, scale,
                             window, sinks, out: torch.Tensor,
                             general: bool = False) -> torch.Tensor:
     """Same attention for one new query per sequence."""
-    if q_lat.numel() and _native_seq(q_lat):
-        _S.latent_attention_decode(out, q_lat, q_rot, cache, block_tables,
+    if q_lat.numel() and _native_lat(q_lat):
+        _L.latent_attention_decode(out, q_lat, q_rot, cache, block_tables,
                                    seq_lens, float(scale), int(window), sinks,
                                    bool(general))
         return out
@@ -675,7 +731,7 @@ def _matrix_core_attention_fits(q: torch.Tensor, k_cache: torch.Tensor,
                                 v_cache: torch.Tensor) -> bool:
     """The llama-class MFMA kernels of ``_C`` take bf16, equal query/key and
     value sizes of 64 or 128 and up to 8 query heads per key head."""
-    if _C is None or _FORCE_REFERENCE or q.dtype != torch.bfloat16:
+    if _attn_ext() is None or _FORCE_REFERENCE or q.dtype != torch.bfloat16:
         return False
     d = q.shape[-1]
     group = q.shape[1] // k_cache.shape[2]
@@ -699,7 +755,7 @@ def gqa_attention_prefill(q, k_cache, v_cache, block_tables, query_start_loc,
     if q.numel() and _native_seq(q):
         if _matrix_core_attention_fits(q, k_cache, v_cache):
             dst = out if out.is_contiguous() else torch.empty_like(q)
-            _C.paged_attention_prefill(dst, q, k_cache, v_cache, block_tables,
+            _attn_ext().paged_attention_prefill(dst, q, k_cache, v_cache, block_tables,
                                        query_start_loc, seq_lens, float(scale),
                                        int(max_query_len))
             if dst is not out:
@@ -722,12 +778,12 @@ def gqa_attention_decode(q, k_cache, v_cache, block_tables, seq_lens, scale,
     if q.numel() and _native_seq(q):
         if _matrix_core_attention_fits(q, k_cache, v_cache):
             if out.is_contiguous():
-                _C.paged_attention_decode(out, q, k_cache, v_cache, block_tables,
-                                          seq_lens, float(scale))
+                _attn_ext().paged_attention_decode(out, q, k_cache, v_cache,
+                                                   block_tables, seq_lens, float(scale))
             else:
                 tmp = torch.empty_like(q)
-                _C.paged_attention_decode(tmp, q, k_cache, v_cache, block_tables,
-                                          seq_lens, float(scale))
+                _attn_ext().paged_attention_decode(tmp, q, k_cache, v_cache,
+                                                   block_tables, seq_lens, float(scale))
                 out.copy_(tmp)
             return out
         _S.paged_attention_any(out, q, k_cache, v_cache, block_tables, None,
