@@ -49,8 +49,8 @@ def layer_norm(x, w, eps):
 
 
 def causal_conv(u, w, b):
-    """u [T, C]; w [C, taps] with the last column on the current token; zeros
-    before the start."""
+    """u [T, C]; column j of w [C, taps] weighs the input taps-1-j steps back;
+    inputs before position 0 count as zero."""
     t, c = u.shape
     taps = w.shape[1]
     out = torch.zeros_like(u)
@@ -153,8 +153,8 @@ def rglru(h, weights, p, m, eps):
 
 
 def mlstm(h, weights, p, m, eps):
-    """Matrix memory with exponential gating and a running maximum that
-    starts at 0."""
+    """Matrix memory with exponential gating, stabilised by a running maximum
+    initialised to 0."""
     t = h.shape[0]
     nh, d, dv, cap = m["heads"], m["dim"], m["vdim"], m["gate_cap"]
     q = (lin(_w(weights, p + "q"), h) * d ** -0.5).view(t, nh, d)

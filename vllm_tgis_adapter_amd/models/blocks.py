@@ -23,7 +23,7 @@ that another design can assemble them differently:
                         per-head scalar decay, gated grouped RMS norm)
 - ``RGLRUMixer``        recurrent block with a real-gated linear recurrent unit
 - ``MLSTMMixer``        matrix memory with exponential gating
-- ``ParallelMixer``     two mixers reading the same input through one merged
+- ``ParallelMixer``     two mixers fed one input through a single merged
                         projection, their outputs mixed with fixed scales
 
 The recurrent mixers keep their state (f32) and the last inputs of their short
@@ -503,8 +503,8 @@ class RGLRUMixer(_Mixer):
 class MLSTMMixer(_Mixer):
     """Matrix memory with exponential gating.  q = W_q h / sqrt(dim), k, v per
     head; log input gate i = cap tanh((W_i h + b) / cap), log forget gate f =
-    logsigmoid(cap tanh((W_f h + b) / cap)); running maximum m (0 at the
-    start): m_t = max(f + m, i), S_t = exp(f + m - m_t) S + exp(i - m_t) k v^T, n
+    logsigmoid(cap tanh((W_f h + b) / cap)); running maximum m, initialised
+    to 0: m_t = max(f + m, i), S_t = exp(f + m - m_t) S + exp(i - m_t) k v^T, n
     likewise with k; o = S^T q / (max(|n . q|, exp(-m_t)) + 1e-6); each head's o
     is RMS-normed, times a weight, times sigmoid(W_g h).  Projected rows:
     [q | k | v | g | i | f]."""
@@ -555,8 +555,8 @@ class MLSTMMixer(_Mixer):
 
 
 class ParallelMixer(nn.Module):
-    """Two mixers side by side on the same input: one merged input projection,
-    result = left_scale * left + right_scale * right.  Returns the two outputs
+    """Two mixers fed one input through a single merged projection; result =
+    left_scale * left + right_scale * right.  Returns the two outputs
     and their scales; the caller's residual kernel forms the sum in f32."""
 
     def __init__(self, width: int, left: _Mixer, right: _Mixer, left_scale: float,

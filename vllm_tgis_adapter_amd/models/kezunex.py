@@ -6,17 +6,17 @@ x <- x + ls2 * LN2b(ff(LN2(x))); every norm is a bias-free layer norm and ls*
 are per-channel layer scales.  The mixer is one of
 
   parallel   grouped-query softmax attention (per-head query/key RMS norm, no
-             rotation, a query temperature that grows with the position) next
-             to a state-space-duality recurrence, both reading the same input,
-             mixed with fixed scales
+             rotation, a query temperature that grows with the position) and a
+             state-space-duality recurrence fed the same normed input, their
+             outputs mixed with fixed scales
   rglru      a recurrent block with a real-gated linear recurrent unit
   mlstm      a matrix memory with exponential gating
 
-``loop`` = {start, stop, times}: layers start..stop-1 run ``times`` times in a
-row with the same weights.  Every pass has cache and state of its own; before
-each pass but the first the embedding output is added to the stream, and
-before each pass the pass's row of ``loop.step`` is.  The output is the model's
-layer norm followed by the embedding table as the head (without its scale).
+``loop`` = {start, stop, times} repeats the layer range [start, stop) ``times``
+times with shared weights; cache and recurrent state are kept per pass.  A pass
+after the first begins by adding the embedding output back into the stream, and
+every pass (the first included) then adds its own row of ``loop.step``.  The
+head is the final layer norm followed by the embedding table, unscaled.
 
 Sizes and constants all come from config.json:
 

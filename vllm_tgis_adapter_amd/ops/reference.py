@@ -534,7 +534,7 @@ def mlstm_scan(
     seq_start_loc, seq_lens, state_slots,
 ) -> torch.Tensor:
     """Matrix memory with exponential gates held stable by a running maximum m
-    (m = 0 before the first token): i = cap * tanh((i_pre + b) / cap), f =
+    (initialised to 0): i = cap * tanh((i_pre + b) / cap), f =
     logsigmoid(cap * tanh((f_pre + b) / cap)), m_t = max(f + m, i), S_t =
     exp(f + m - m_t) S + exp(i - m_t) k v^T, n_t likewise with k, o = S_t^T q /
     (max(|n_t . q|, exp(-m_t)) + 1e-6).  Returns o [T, H*vdim] f32."""
