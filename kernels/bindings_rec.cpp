@@ -33,13 +33,14 @@ void launch_paged_attention_any(T*, long, const T*, long, const T*, const T*,
 template <typename T>
 void launch_ssd_scan(float*, const T*, long, const T*, long, const float*,
                      const float*, const float*, float*, const int*, const int*,
-                     const int*, int, int, int, int, int, int, hipStream_t);
+                     const int*, int, int, int, int, int, int, float*, int,
+                     hipStream_t);
 template <typename T>
 void launch_mlstm_scan(float*, const T*, long, const T*, long, const T*, long,
                        const T*, long, const T*, long, const float*,
                        const float*, float, float, float*, float*, float*,
                        const int*, const int*, const int*, int, int, int, int,
-                       int, hipStream_t);
+                       int, float*, int, hipStream_t);
 template <typename T>
 void launch_rglru_scan(T*, const T*, const T*, const T*, const float*,
                        const float*, const float*, float, const T*, float*,
@@ -310,13 +311,15 @@ void ssd_scan(torch::Tensor y, torch::Tensor xbc, torch::Tensor dt,
   if (rows == 0 || nseq == 0) return;
   const int vec_ok = nstate % 8 == 0 && inner % 8 == 0 && xbc.stride(0) % 8 == 0 &&
                      aligned16(xbc) && aligned16(state);
+  // alpha, beta per (row, head), written by the gate kernel ahead of the scan
+  auto gates = torch::empty({(long)rows * heads * 4}, y.options());
   DISPATCH_F32_BF16(xbc.scalar_type(), {
     launch_ssd_scan<scalar_t>(
         ptr<float>(y), ptr<scalar_t>(xbc), (long)xbc.stride(0), ptr<scalar_t>(dt),
         (long)dt.stride(0), ptr<float>(dt_bias), ptr<float>(a_log),
         ptr<float>(d_skip), ptr<float>(state), ptr<int>(loc), ptr<int>(seq_lens),
         ptr<int>(slots), nseq, (int)heads, (int)vdim, (int)nstate, (int)groups,
-        vec_ok, stream());
+        vec_ok, ptr<float>(gates), rows, stream());
   });
 }
 
@@ -360,6 +363,8 @@ void mlstm_scan(torch::Tensor o, torch::Tensor q, torch::Tensor k, torch::Tensor
   const int vec_ok = dim % 8 == 0 && q.stride(0) % 8 == 0 && k.stride(0) % 8 == 0 &&
                      aligned16(q) && aligned16(k) && aligned16(s_state) &&
                      aligned16(n_state);
+  // alpha, beta, exp(-m) per (row, head), written by the gate kernels
+  auto gates = torch::empty({(long)rows * heads * 4}, o.options());
   DISPATCH_F32_BF16(dt, {
     launch_mlstm_scan<scalar_t>(
         ptr<float>(o), ptr<scalar_t>(q), (long)q.stride(0), ptr<scalar_t>(k),
@@ -368,7 +373,7 @@ void mlstm_scan(torch::Tensor o, torch::Tensor q, torch::Tensor k, torch::Tensor
         (long)f_pre.stride(0), ptr<float>(i_bias), ptr<float>(f_bias), (float)cap,
         (float)q_scale, ptr<float>(s_state), ptr<float>(n_state),
         ptr<float>(m_state), ptr<int>(loc), ptr<int>(seq_lens), ptr<int>(slots),
-        nseq, heads, dim, vdim, vec_ok, stream());
+        nseq, heads, dim, vdim, vec_ok, ptr<float>(gates), rows, stream());
   });
 }
 

@@ -17,6 +17,9 @@
 //   KIND_MLSTM  log gates i, f (capped), running maximum m: alpha = exp(f + m
 //               - m'), beta = exp(i - m'), a normaliser n_t = alpha n + beta k,
 //               y = S q / (max(|n . q|, exp(-m')) + 1e-6)
+// alpha, beta (and exp(-m')) are computed once per (row, head) by small gate
+// kernels ahead of the scan (for the mLSTM a sequential pass over the rows
+// carries the maximum), not by every thread of it.
 // The N axis is split over NSP adjacent lanes, 16 state values per lane in
 // registers (N <= 1024); a workgroup of 256 threads owns 256 / NSP value
 // columns of one (sequence, head), or four times as many with four columns
@@ -67,12 +70,62 @@ struct ScanArgs {
   long g0_st, g1_st;
   const float* p0; const float* p1; const float* p2;  // SSD: dt_bias, A_log, D; mLSTM: i_bias, f_bias
   float cap, q_scale;
+  float4* gates; int rows;           // per (row, head): alpha, beta, exp(-m), -  (f32)
   float* y; long y_st;               // [T, H*vdim] f32
   float* s_state; float* n_state; float* m_state;
   const int* loc; const int* seq_lens; const int* slots;
   int heads, vdim, nk, per_group;    // nk = N (SSD) or dim (mLSTM); heads per k/q group
   int vec_ok;
 };
+
+// Gates per (row, head), computed once instead of by every thread of the scan.
+// Pointwise part: SSD alpha = exp(-exp(A_log) dt), beta = dt; mLSTM the capped
+// log gates (i in .x, f in .y) that the sequential pass below turns into
+// alpha, beta and exp(-m).
+template <typename T, int KIND>
+__global__ void scan_gates_pointwise_kernel(ScanArgs a) {
+  const long idx = blockIdx.x * (long)blockDim.x + threadIdx.x;
+  if (idx >= (long)a.rows * a.heads) return;
+  const long row = idx / a.heads;
+  const int h = (int)(idx - row * a.heads);
+  const float g0 = ScalarOps<T>::to_f32(reinterpret_cast<const T*>(a.g0)[row * a.g0_st + h]);
+  float4 out = make_float4(0.f, 0.f, 1.f, 0.f);
+  if (KIND == KIND_SSD) {
+    const float dt = softplus_f(g0 + a.p0[h]);
+    out.x = expf(-expf(a.p1[h]) * dt);
+    out.y = dt;
+  } else {
+    const float g1 = ScalarOps<T>::to_f32(reinterpret_cast<const T*>(a.g1)[row * a.g1_st + h]);
+    out.x = a.cap * tanhf((g0 + a.p0[h]) / a.cap);
+    out.y = logsigmoid_f(a.cap * tanhf((g1 + a.p1[h]) / a.cap));
+  }
+  a.gates[idx] = out;
+}
+
+// mLSTM: one thread per (sequence, head) walks the step's rows with the
+// running maximum (0 at position 0): m' = max(f + m, i), alpha = exp(f + m -
+// m'), beta = exp(i - m'), and stores exp(-m') for the output's denominator.
+// Leaves the new maximum in m_state; nothing else reads m_state in the step.
+__global__ void mlstm_gates_scan_kernel(ScanArgs a, int nseq) {
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= nseq * a.heads) return;
+  const int s = idx / a.heads;
+  const int h = idx - s * a.heads;
+  const int row0 = a.loc[s];
+  const int n = a.loc[s + 1] - row0;
+  const int slot = a.slots[s];
+  if (n <= 0 || slot < 0) return;
+  float* mp = a.m_state + (long)slot * a.heads + h;
+  float m = (a.seq_lens[s] - n) > 0 ? *mp : 0.f;
+  for (int r = 0; r < n; ++r) {
+    float4* g = a.gates + (long)(row0 + r) * a.heads + h;
+    const float ig = g->x, fg = g->y;
+    const float m_new = fmaxf(fg + m, ig);
+    *g = make_float4(expf(fg + m - m_new), expf(ig - m_new), expf(-m_new), 0.f);
+    m = m_new;
+  }
+  *mp = m;
+}
 
 template <typename T, int KIND, int NSP, int VPT>
 __global__ __launch_bounds__(256) void matrix_scan_kernel(ScanArgs a) {
@@ -105,16 +158,12 @@ __global__ __launch_bounds__(256) void matrix_scan_kernel(ScanArgs a) {
   for (int c = 0; c < VPT; ++c) jc[c] = min(jbase + c, a.vdim - 1);
 
   float S[VPT][NPT], nst[NPT];
-  float m = 0.f;
   float* sbase = a.s_state + ((long)slot * a.heads + h) * a.vdim * a.nk;
   const float* nrow = KIND == KIND_MLSTM ? a.n_state + ((long)slot * a.heads + h) * a.nk : nullptr;
   if (start > 0) {
 #pragma unroll
     for (int c = 0; c < VPT; ++c) load_slice<float>(sbase + (long)jc[c] * a.nk, n0, a.nk, vec, S[c]);
-    if (KIND == KIND_MLSTM) {
-      load_slice<float>(nrow, n0, a.nk, vec, nst);
-      m = a.m_state[(long)slot * a.heads + h];
-    }
+    if (KIND == KIND_MLSTM) load_slice<float>(nrow, n0, a.nk, vec, nst);
   } else {
 #pragma unroll
     for (int i = 0; i < NPT; ++i) {
@@ -124,20 +173,11 @@ __global__ __launch_bounds__(256) void matrix_scan_kernel(ScanArgs a) {
     }
   }
 
-  float c0 = 0.f, c1 = 0.f, c2 = 0.f;
-  if (KIND == KIND_SSD) {
-    c0 = a.p0[h];               // dt bias
-    c1 = -expf(a.p1[h]);        // -A
-    c2 = a.p2[h];               // D
-  } else {
-    c0 = a.p0[h];               // input-gate bias
-    c1 = a.p1[h];               // forget-gate bias
-  }
+  const float c2 = KIND == KIND_SSD ? a.p2[h] : 0.f;   // D
+  const float4* gp = a.gates + h;
   const T* qp = reinterpret_cast<const T*>(a.q) + (long)grp * a.nk;
   const T* kp = reinterpret_cast<const T*>(a.k) + (long)grp * a.nk;
   const T* vp = reinterpret_cast<const T*>(a.v) + (long)h * a.vdim;
-  const T* g0 = reinterpret_cast<const T*>(a.g0) + h;
-  const T* g1 = KIND == KIND_MLSTM ? reinterpret_cast<const T*>(a.g1) + h : nullptr;
 
   for (int r = 0; r < n; ++r) {
     const long row = row0 + r;
@@ -146,41 +186,28 @@ __global__ __launch_bounds__(256) void matrix_scan_kernel(ScanArgs a) {
     load_slice<T>(qp + row * a.q_st, n0, a.nk, vec, qq);
 #pragma unroll
     for (int c = 0; c < VPT; ++c) vj[c] = ScalarOps<T>::to_f32(vp[row * a.v_st + jc[c]]);
-    float alpha, beta;
-    if (KIND == KIND_SSD) {
-      const float dt = softplus_f(ScalarOps<T>::to_f32(g0[row * a.g0_st]) + c0);
-      alpha = expf(c1 * dt);
-      beta = dt;
-    } else {
-      const float ig = a.cap * tanhf((ScalarOps<T>::to_f32(g0[row * a.g0_st]) + c0) / a.cap);
-      const float fg = logsigmoid_f(
-          a.cap * tanhf((ScalarOps<T>::to_f32(g1[row * a.g1_st]) + c1) / a.cap));
-      const float m_new = fmaxf(fg + m, ig);
-      alpha = expf(fg + m - m_new);
-      beta = expf(ig - m_new);
-      m = m_new;
-    }
+    const float4 gt = gp[row * a.heads];
+    const float alpha = gt.x, beta = gt.y;
     float dot[VPT], ndot = 0.f;
 #pragma unroll
     for (int c = 0; c < VPT; ++c) dot[c] = 0.f;
 #pragma unroll
     for (int i = 0; i < NPT; ++i) {
       const float bk = beta * kk[i];
-      const float qs = KIND == KIND_MLSTM ? qq[i] * a.q_scale : qq[i];
       if (KIND == KIND_MLSTM) {
         nst[i] = alpha * nst[i] + bk;
-        ndot += nst[i] * qs;
+        ndot += nst[i] * qq[i];
       }
 #pragma unroll
       for (int c = 0; c < VPT; ++c) {
         S[c][i] = alpha * S[c][i] + bk * vj[c];
-        dot[c] += S[c][i] * qs;
+        dot[c] += S[c][i] * qq[i];
       }
     }
-    float den = 1.f;
+    float den = 1.f;    // mLSTM: the query scale is applied to the two sums
     if (KIND == KIND_MLSTM) {
-      ndot = group_reduce_sum<NSP>(ndot);
-      den = 1.0f / (fmaxf(fabsf(ndot), expf(-m)) + 1e-6f);
+      ndot = group_reduce_sum<NSP>(ndot) * a.q_scale;
+      den = a.q_scale / (fmaxf(fabsf(ndot), gt.z) + 1e-6f);
     }
 #pragma unroll
     for (int c = 0; c < VPT; ++c) {
@@ -206,13 +233,13 @@ __global__ __launch_bounds__(256) void matrix_scan_kernel(ScanArgs a) {
         if (n0 + i < a.nk) srow[n0 + i] = S[c][i];
     }
   }
-  // the normaliser n and the maximum m are read by every workgroup of this
-  // (sequence, head) and therefore advanced by a kernel of their own, after
-  // this one, on the same stream
+  // the normaliser n is read by every workgroup of this (sequence, head) and
+  // therefore advanced by a kernel of its own, after this one, on the same
+  // stream
 }
 
-// Advances n [slots, H, dim] and m [slots, H] of the mLSTM over the step's
-// rows: one workgroup per (sequence, head), one thread per key dim.
+// Advances the mLSTM normaliser n [slots, H, dim] over the step's rows with the
+// precomputed gates: one workgroup per (sequence, head), one thread per key dim.
 template <typename T>
 __global__ __launch_bounds__(256) void mlstm_norm_state_kernel(ScanArgs a) {
   const int s = blockIdx.x / a.heads;
@@ -222,33 +249,18 @@ __global__ __launch_bounds__(256) void mlstm_norm_state_kernel(ScanArgs a) {
   const int slot = a.slots[s];
   if (n <= 0 || slot < 0) return;
   const int start = a.seq_lens[s] - n;
-  const float c0 = a.p0[h], c1 = a.p1[h];
   const T* kp = reinterpret_cast<const T*>(a.k) + (long)h * a.nk;
-  const T* g0 = reinterpret_cast<const T*>(a.g0) + h;
-  const T* g1 = reinterpret_cast<const T*>(a.g1) + h;
+  const float4* gp = a.gates + h;
   float* nrow = a.n_state + ((long)slot * a.heads + h) * a.nk;
-  float* mp = a.m_state + (long)slot * a.heads + h;
-  const float m0 = start > 0 ? *mp : 0.f;
-  float m = m0;
-  for (int d = threadIdx.x; d < a.nk || d == threadIdx.x; d += blockDim.x) {
-    const bool ok = d < a.nk;
-    float nv = (ok && start > 0) ? nrow[d] : 0.f;
-    m = m0;
+  for (int d = threadIdx.x; d < a.nk; d += blockDim.x) {
+    float nv = start > 0 ? nrow[d] : 0.f;
     for (int r = 0; r < n; ++r) {
       const long row = row0 + r;
-      const float ig = a.cap * tanhf((ScalarOps<T>::to_f32(g0[row * a.g0_st]) + c0) / a.cap);
-      const float fg = logsigmoid_f(
-          a.cap * tanhf((ScalarOps<T>::to_f32(g1[row * a.g1_st]) + c1) / a.cap));
-      const float m_new = fmaxf(fg + m, ig);
-      const float kv = ok ? ScalarOps<T>::to_f32(kp[row * a.k_st + d]) : 0.f;
-      nv = expf(fg + m - m_new) * nv + expf(ig - m_new) * kv;
-      m = m_new;
+      const float4 gt = gp[row * a.heads];
+      nv = gt.x * nv + gt.y * ScalarOps<T>::to_f32(kp[row * a.k_st + d]);
     }
-    if (ok) nrow[d] = nv;
+    nrow[d] = nv;
   }
-  // every thread read the old maximum before this barrier
-  __syncthreads();
-  if (threadIdx.x == 0) *mp = m;
 }
 
 template <typename T, int KIND>
@@ -323,9 +335,11 @@ void launch_ssd_scan(float* y, const T* xbc, long xbc_st, const T* dt, long dt_s
                      const float* dt_bias, const float* a_log, const float* d_skip,
                      float* state, const int* loc, const int* seq_lens,
                      const int* slots, int nseq, int heads, int vdim, int nstate,
-                     int groups, int vec_ok, hipStream_t stream) {
+                     int groups, int vec_ok, float* gates, int rows,
+                     hipStream_t stream) {
   const int inner = heads * vdim;
   ScanArgs a{};
+  a.gates = reinterpret_cast<float4*>(gates); a.rows = rows;
   a.v = xbc;                                  a.v_st = xbc_st;
   a.k = xbc + inner;                          a.k_st = xbc_st;
   a.q = xbc + inner + (long)groups * nstate;  a.q_st = xbc_st;
@@ -336,6 +350,8 @@ void launch_ssd_scan(float* y, const T* xbc, long xbc_st, const T* dt, long dt_s
   a.loc = loc; a.seq_lens = seq_lens; a.slots = slots;
   a.heads = heads; a.vdim = vdim; a.nk = nstate; a.per_group = heads / groups;
   a.vec_ok = vec_ok;
+  const long ng = (long)rows * heads;
+  scan_gates_pointwise_kernel<T, KIND_SSD><<<(int)((ng + 255) / 256), 256, 0, stream>>>(a);
   launch_matrix_scan<T, KIND_SSD>(a, nseq, stream);
 }
 
@@ -347,8 +363,9 @@ void launch_mlstm_scan(float* o, const T* q, long q_st, const T* k, long k_st,
                        float* s_state, float* n_state, float* m_state,
                        const int* loc, const int* seq_lens, const int* slots,
                        int nseq, int heads, int dim, int vdim, int vec_ok,
-                       hipStream_t stream) {
+                       float* gates, int rows, hipStream_t stream) {
   ScanArgs a{};
+  a.gates = reinterpret_cast<float4*>(gates); a.rows = rows;
   a.q = q; a.q_st = q_st; a.k = k; a.k_st = k_st; a.v = v; a.v_st = v_st;
   a.g0 = i_pre; a.g0_st = i_st; a.g1 = f_pre; a.g1_st = f_st;
   a.p0 = i_bias; a.p1 = f_bias;
@@ -358,6 +375,9 @@ void launch_mlstm_scan(float* o, const T* q, long q_st, const T* k, long k_st,
   a.loc = loc; a.seq_lens = seq_lens; a.slots = slots;
   a.heads = heads; a.vdim = vdim; a.nk = dim; a.per_group = 1;
   a.vec_ok = vec_ok;
+  const long ng = (long)rows * heads;
+  scan_gates_pointwise_kernel<T, KIND_MLSTM><<<(int)((ng + 255) / 256), 256, 0, stream>>>(a);
+  mlstm_gates_scan_kernel<<<(nseq * heads + 63) / 64, 64, 0, stream>>>(a, nseq);
   launch_matrix_scan<T, KIND_MLSTM>(a, nseq, stream);
   const int block = dim >= 256 ? 256 : ((dim + 63) / 64) * 64;
   mlstm_norm_state_kernel<T><<<nseq * heads, block, 0, stream>>>(a);
@@ -380,12 +400,13 @@ void launch_rglru_scan(T* out, const T* u, const T* r_pre, const T* i_pre,
   template void launch_ssd_scan<T>(float*, const T*, long, const T*, long,      \
                                    const float*, const float*, const float*,    \
                                    float*, const int*, const int*, const int*,  \
-                                   int, int, int, int, int, int, hipStream_t);  \
+                                   int, int, int, int, int, int, float*, int,   \
+                                   hipStream_t);                                \
   template void launch_mlstm_scan<T>(                                           \
       float*, const T*, long, const T*, long, const T*, long, const T*, long,   \
       const T*, long, const float*, const float*, float, float, float*, float*, \
       float*, const int*, const int*, const int*, int, int, int, int, int,      \
-      hipStream_t);                                                             \
+      float*, int, hipStream_t);                                                \
   template void launch_rglru_scan<T>(T*, const T*, const T*, const T*,          \
                                      const float*, const float*, const float*,  \
                                      float, const T*, float*, const int*,       \
