@@ -549,7 +549,7 @@ def _kezunex_model_config(name: str, sz: dict, dtype: str):
                   "norm_groups": 1},
         "left_scale": 0.5, "right_scale": 0.5}}
     mls = {"type": "mlstm", "mlp": None,
-           "mixer": {"heads": mh, "dim": md, "vdim": mv, "gate_cap": 15.0}}
+           "mixer": {"heads": mh, "dim": md, "vdim": mv, "gate_cap": 12.0}}
     rec = {"type": "rglru", "mlp": None, "mixer": {"width": rw, "blocks": rb, "conv": 4}}
     n = sz["layers"]
     # looped [mlstm, parallel] x 2, then rglru / parallel alternating

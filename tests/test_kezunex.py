@@ -376,7 +376,7 @@ def test_matrix_core_shapes(tmp_path, device, dtype):
     L = oracle.layer
     cfg = oracle.make_config(
         width=128, vocab=211,
-        layers=[L("parallel", ff=128, left=oracle.attn_spec(4, 2, 64, 64, 0.1, 0.5, 32),
+        layers=[L("parallel", ff=128, left=oracle.attn_spec(4, 2, 64, 64, 0.1, 0.3, 32),
                   right=oracle.ssd_spec(4, 32, 64, 1, 4, 1)),
                 L("mlstm", heads=2, dim=32, vdim=64)],
         loop=(0, 1, 2))
@@ -429,6 +429,35 @@ def test_captured_decode_steps_match_eager(model):
         _close(outs[1][k], want)
         _close(outs[0][k], outs[1][k])
     _close(outs[1]["c"], oracle.forward(cfg, w, toks["c"])[:22])
+
+
+@pytest.mark.gpu
+def test_captured_decode_with_padding_rows(model):
+    """Three sequences decode together in the four-row captured bucket: the
+    padding row (slot -1, length 0) must leave every state slot alone."""
+    cfg, w, path = model
+    toks = {k: _tokens(n, cfg["vocab"], 70 + i) for i, (k, n) in
+            enumerate([("a", 14), ("b", 11), ("c", 12), ("d", 9)])}
+    e = _engine(path, "cuda", blocks=32, slots=4, eager=False)
+    assert 4 in e.worker.graph_runner.graphs
+    got = {k: [] for k in toks}
+    at = {k: 0 for k in toks}
+
+    def step(parts, done=()):
+        entries = [(k, toks[k][at[k]:at[k] + n], list(range(n))) for k, n in parts]
+        lg = e.replay_step(entries, list(done)).double().cpu()
+        o = 0
+        for k, n in parts:
+            got[k].append(lg[o:o + n])
+            at[k] += n
+            o += n
+
+    step([("a", 5), ("b", 3), ("c", 4), ("d", 9)], done=["d"])   # d's slot is dirty now
+    for _ in range(6):
+        step([("a", 1), ("b", 1), ("c", 1)])                     # bucket 4, one padding row
+    step([("a", 3), ("b", 2), ("c", 2)], done=["a", "b", "c"])
+    for k in ("a", "b", "c", "d"):
+        _close(torch.cat(got[k]), oracle.forward(cfg, w, toks[k]), what=k)
 
 
 @pytest.mark.parametrize("device", DEVICES)
