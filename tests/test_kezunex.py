@@ -370,13 +370,16 @@ def test_bf16_stays_near_oracle(model, device):
 
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_matrix_core_shapes(tmp_path, device, dtype):
+@pytest.mark.parametrize("attn", [(4, 2, 64), (6, 2, 128), (8, 1, 64), (3, 3, 128)])
+def test_matrix_core_shapes(tmp_path, device, dtype, attn):
     """Head sizes the MFMA attention kernels take (bf16, key size = value size
-    = 64) and vector-width state sizes."""
+    of 64 or 128, one to eight query heads per key head) and vector-width
+    state sizes."""
     L = oracle.layer
+    nh, ng, hd = attn
     cfg = oracle.make_config(
         width=128, vocab=211,
-        layers=[L("parallel", ff=128, left=oracle.attn_spec(4, 2, 64, 64, 0.1, 0.3, 32),
+        layers=[L("parallel", ff=128, left=oracle.attn_spec(nh, ng, hd, hd, 0.1, 0.3, 32),
                   right=oracle.ssd_spec(4, 32, 64, 1, 4, 1)),
                 L("mlstm", heads=2, dim=32, vdim=64)],
         loop=(0, 1, 2))
