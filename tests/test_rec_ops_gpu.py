@@ -92,7 +92,7 @@ def test_gated_group_norm(dtype, gate_first):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("dims", [(5, 5, 24, 40), (6, 2, 32, 32), (4, 1, 72, 16), (3, 3, 10, 6),
-                                  (8, 2, 128, 128), (2, 1, 256, 64)])
+                                  (8, 2, 128, 128), (2, 1, 256, 64), (2, 1, 32, 320), (1, 1, 8, 1000)])
 def test_qk_norm_and_attention(dtype, dims):
     heads, kvh, dim, vdim = dims
     g = torch.Generator().manual_seed(3)

@@ -157,7 +157,7 @@ def topk_softmax(gate_logits: torch.Tensor, top_k: int) -> tuple[torch.Tensor, t
 
 # ---------------------------------------------------------------------------
 # f32 residual-stream ops, short causal convolution with per-sequence state,
-# windowed latent attention with sinks (the `_C_seq` kernel set)
+# windowed latent attention with sinks (the `_C_seq` and `_C_lat` kernel sets)
 # ---------------------------------------------------------------------------
 
 
