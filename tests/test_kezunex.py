@@ -539,3 +539,44 @@ def test_refuses_what_it_cannot_run(tmp_path):
     path = oracle.save_model(tmp_path / "bad", cfg, {})
     with pytest.raises(ValueError):
         _engine(path, "cpu")
+
+
+def test_trace_replay_program(tmp_path):
+    """bin/trace_run as a user runs it: JSON steps on stdin, 'done <step>' lines
+    on stdout, little-endian f32 logits files for the steps that want some;
+    two requests in portions side by side, one leaving early."""
+    import json
+    import os
+    import subprocess
+    import sys
+
+    import numpy as np
+
+    cfg = oracle.make_config()
+    w = oracle.make_weights(cfg, seed=8)
+    path = oracle.save_model(tmp_path / "m", cfg, w)
+    a, b = _tokens(70, cfg["vocab"], 41), _tokens(9, cfg["vocab"], 42)
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": a[:66], "want": [0, 65]}], "end": []},
+        {"step": 1, "entries": [{"id": "b", "tokens": b[:2], "want": []}], "end": []},
+        {"step": 2, "entries": [{"id": "a", "tokens": a[66:67], "want": [0]},
+                                {"id": "b", "tokens": b[2:], "want": [6, 2]}], "end": ["b"]},
+        {"step": 3, "entries": [{"id": "a", "tokens": a[67:], "want": [2, 0]}], "end": ["a"]},
+    ]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = tmp_path / "out"
+    proc = subprocess.run(
+        [sys.executable, os.path.join(root, "bin", "trace_run"), "--model", path, "--dtype",
+         "float32", "--out", str(out), "--max-tokens", "192", "--device", "cpu"],
+        input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True,
+        timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    done = [ln for ln in proc.stdout.splitlines() if ln.startswith("done ")]
+    assert done == ["done 0", "done 1", "done 2", "done 3"]
+    assert not (out / "1.f32").exists()
+    wa, wb = oracle.forward(cfg, w, a), oracle.forward(cfg, w, b)
+    want = {0: torch.stack([wa[0], wa[65]]), 2: torch.stack([wa[66], wb[8], wb[4]]),
+            3: torch.stack([wa[69], wa[67]])}
+    for n, rows in want.items():
+        got = np.fromfile(out / f"{n}.f32", dtype="<f4").reshape(-1, cfg["vocab"])
+        _close(torch.from_numpy(got).double(), rows, what=f"step {n}")
