@@ -26,7 +26,8 @@
 // per thread (the key / query slices a thread loads then serve four columns).  State rows are stored [vdim, N] so that a
 // wave loads and stores them as one contiguous run.  The value columns are
 // independent of each other, so there is no barrier in the token loop: per
-// token a thread does 32 FMAs and log2(NSP) shuffles for the dot product.
+// token a thread does 32 FMAs per column and log2(NSP) DPP adds for its dot
+// product.
 //
 // rglru_scan: elementwise linear recurrence, one thread per (sequence,
 // channel), gates and decay computed in f32 on the fly.
@@ -41,6 +42,27 @@ enum { KIND_SSD = 0, KIND_MLSTM = 1 };
 DEVINLINE float softplus_f(float x) { return fmaxf(x, 0.f) + log1pf(expf(-fabsf(x))); }
 DEVINLINE float logsigmoid_f(float x) { return fminf(x, 0.f) - log1pf(expf(-fabsf(x))); }
 DEVINLINE float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+// Sum over NSP adjacent lanes (NSP a power of two, groups aligned), result in
+// every lane.  Up to 16 lanes the partner values come through DPP modifiers on
+// the adds (quad permutes, then the half-row and row mirrors — each mirror
+// pairs a lane with one from the other, already uniform, half), which costs no
+// LDS-crossbar round trip; wider groups finish with two shuffles.
+template <int CTRL>
+DEVINLINE float dpp_move(float v) {
+  return __int_as_float(
+      __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+template <int NSP>
+DEVINLINE float lanes_sum(float x) {
+  if (NSP >= 2) x += dpp_move<0xB1>(x);    // quad_perm [1,0,3,2]
+  if (NSP >= 4) x += dpp_move<0x4E>(x);    // quad_perm [2,3,0,1]
+  if (NSP >= 8) x += dpp_move<0x141>(x);   // row_half_mirror
+  if (NSP >= 16) x += dpp_move<0x140>(x);  // row_mirror
+  if (NSP >= 32) x += __shfl_xor(x, 16, WAVE_SIZE);
+  if (NSP >= 64) x += __shfl_xor(x, 32, WAVE_SIZE);
+  return x;
+}
 
 // 16 consecutive values p[n0 .. n0+16) of a row of length n_total as f32,
 // zeros past the end
@@ -206,12 +228,12 @@ __global__ __launch_bounds__(256) void matrix_scan_kernel(ScanArgs a) {
     }
     float den = 1.f;    // mLSTM: the query scale is applied to the two sums
     if (KIND == KIND_MLSTM) {
-      ndot = group_reduce_sum<NSP>(ndot) * a.q_scale;
+      ndot = lanes_sum<NSP>(ndot) * a.q_scale;
       den = a.q_scale / (fmaxf(fabsf(ndot), gt.z) + 1e-6f);
     }
 #pragma unroll
     for (int c = 0; c < VPT; ++c) {
-      const float d = group_reduce_sum<NSP>(dot[c]);
+      const float d = lanes_sum<NSP>(dot[c]);
       const float yv = KIND == KIND_MLSTM ? d * den : d + c2 * vj[c];
       if (ns == 0 && jbase + c < a.vdim)
         a.y[row * a.y_st + (long)h * a.vdim + jbase + c] = yv;
